@@ -1,0 +1,171 @@
+/*
+ * libleanffn -- C ABI of the MI355X (gfx950) LeanFFN kernels.
+ *
+ * Everything here takes plain device pointers and sizes.  The library never allocates or frees device memory, keeps no
+ * pointer after a call returns, launches asynchronously on the stream it is given and never synchronises.  Every function
+ * that returns int returns LT_OK (0) or an lt_status error; lt_last_error() gives the message for the calling thread.
+ * No C++ exception crosses this boundary.
+ *
+ * Reference interfaces replaced (paths relative to the learning-at-home/lean_transformer checkout):
+ *   lt_ffn_forward / lt_ffn_backward   _LeanFFN.forward  lean_transformer/ffn.py:146-217,
+ *                                      _LeanFFN.backward lean_transformer/ffn.py:233-306
+ *   lt_linear_forward / _backward      _GeneralizedLinear.forward_functional / backward_functional
+ *                                      lean_transformer/blocksparse/linear.py:161-230, :237-328
+ *   lt_blocksparse_forward / _backward blocksparse_matmul / blocksparse_matmul_backward
+ *                                      lean_transformer/blocksparse/native_backend.py:9-35, :38-76
+ *                                      (also the role of the matmul_op plug-in slot, blocksparse/triton_backend.py:37-79)
+ *   lt_layernorm_forward / _backward   the F.layer_norm calls and their autograd, lean_transformer/ffn.py:184,283,290-293
+ *   lt_activation_forward / _backward  gelu_fused / gelu_fused_grad lean_transformer/utils.py:24-38 and
+ *                                      _LeanFFN._apply_activation   lean_transformer/ffn.py:138-144
+ *   lt_dropout_mask                    the mask torch.dropout draws at lean_transformer/ffn.py:204 and replays at :245
+ */
+#ifndef LEANFFN_H
+#define LEANFFN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum lt_status {
+  LT_OK = 0,
+  LT_ERR_BAD_ARG = 1,     /* null pointer, non-positive size, misaligned pointer */
+  LT_ERR_UNSUPPORTED = 2, /* a combination the kernels do not implement */
+  LT_ERR_WORKSPACE = 3,   /* workspace smaller than lt_*_workspace_bytes() */
+  LT_ERR_HIP = 4          /* a HIP runtime call or kernel launch failed */
+} lt_status;
+
+typedef enum lt_dtype { LT_F32 = 0, LT_BF16 = 1 } lt_dtype;
+
+typedef enum lt_act { LT_ACT_GELU_FUSED = 0, LT_ACT_GELU = 1, LT_ACT_RELU = 2, LT_ACT_SILU = 3 } lt_act;
+
+/* One projection in the reference's "generalized linear" form: main weight (dense or native block-sparse), optional bias,
+ * optional low-rank pair.  Weights and low-rank factors are in the compute dtype; the bias is always fp32. */
+typedef struct lt_linear {
+  const void* weight;              /* dense: [out_features, in_features]; sparse: [in_features, blocks_per_in, block] */
+  const float* bias;               /* [out_features] or NULL */
+  const void* lowrank_first;       /* [lowrank, in_features] or NULL */
+  const void* lowrank_second;      /* [out_features, lowrank] or NULL */
+  const int32_t* forward_indices;  /* sparse: [out_features / block, blocks_per_out]; dense: NULL */
+  const int64_t* backward_indices; /* sparse: [in_features / block, blocks_per_in]; dense: NULL */
+  int32_t in_features;
+  int32_t out_features;
+  int32_t lowrank;        /* 0 when there is no low-rank term */
+  int32_t block;          /* sparse block size, 0 when dense */
+  int32_t blocks_per_out; /* K: active blocks per output block row */
+  int32_t blocks_per_in;  /* A: active blocks per input block column */
+} lt_linear;
+
+/* Where lt_linear_backward / lt_ffn_backward write parameter gradients; a NULL member skips that gradient.
+ * weight / lowrank_* are in the compute dtype and shaped like the parameter, bias is fp32. */
+typedef struct lt_linear_grads {
+  void* weight;
+  float* bias;
+  void* lowrank_first;
+  void* lowrank_second;
+} lt_linear_grads;
+
+typedef struct lt_ffn_desc {
+  int64_t tokens;       /* T: rows of the flattened input */
+  int32_t hidden;       /* H */
+  int32_t intermediate; /* I; the up-projection has 2*I outputs when gated (first half = gate) */
+  int32_t gated;
+  int32_t act;           /* lt_act */
+  int32_t residual;      /* add the input to the output */
+  int32_t io_dtype;      /* lt_dtype of x, y, dy, dx */
+  int32_t compute_dtype; /* lt_dtype of weights, GEMM operands, the saved pre-activation and weight gradients */
+  float ln_eps;
+  float dropout_p;        /* 0 disables dropout (also pass 0 in eval mode) */
+  uint64_t dropout_seed;  /* Philox key */
+  uint64_t dropout_offset;/* Philox stream offset; forward and backward of one call must pass the same pair */
+  const float* ln_weight; /* [H] fp32 */
+  const float* ln_bias;   /* [H] fp32 */
+  const float* post_ln_weight; /* [H] fp32 or NULL: optional LayerNorm after the down-projection */
+  const float* post_ln_bias;
+  lt_linear i2h; /* H -> (gated ? 2I : I) */
+  lt_linear h2o; /* I -> H */
+} lt_ffn_desc;
+
+/* Activations kept between forward and backward (all caller-allocated).  This is the reference's save-set
+ * (lean_transformer/ffn.py:210-216) plus the LayerNorm row statistics (8 bytes per token). */
+typedef struct lt_ffn_saved {
+  void* pre_activation;  /* [T, 2I or I] compute dtype */
+  float* ln_stats;       /* [T, 2] (mean, rstd) of the pre-LayerNorm */
+  void* post_ln_input;   /* [T, H] compute dtype; only with post-LN, else NULL */
+  void* i2h_lowrank_hid; /* [T, i2h.lowrank] compute dtype or NULL */
+  void* h2o_lowrank_hid; /* [T, h2o.lowrank] compute dtype or NULL */
+} lt_ffn_saved;
+
+typedef struct lt_ffn_grads {
+  void* dx;               /* [T, H] io dtype, or NULL */
+  float* ln_weight;       /* [H] fp32 (both or neither of ln_weight / ln_bias) */
+  float* ln_bias;
+  float* post_ln_weight;
+  float* post_ln_bias;
+  lt_linear_grads i2h;
+  lt_linear_grads h2o;
+} lt_ffn_grads;
+
+const char* lt_version(void);
+const char* lt_last_error(void);
+
+/* ---- whole FFN block ------------------------------------------------------------------------------------------------ */
+size_t lt_ffn_forward_workspace_bytes(const lt_ffn_desc* desc);
+size_t lt_ffn_backward_workspace_bytes(const lt_ffn_desc* desc);
+/* y = [x +] dropout([postLN](act(LN(x) W1^T + b1) W2^T + b2)); fills *saved. */
+int lt_ffn_forward(const lt_ffn_desc* desc, const void* x, void* y, const lt_ffn_saved* saved, void* workspace,
+                   size_t workspace_bytes, void* stream);
+/* gradients of the above given dy, recomputing LayerNorm output and activation from x and saved->pre_activation */
+int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const void* dy, const lt_ffn_saved* saved,
+                    const lt_ffn_grads* grads, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- generalized linear: y = x W^T (+ bias) (+ (x L1^T) L2^T) ------------------------------------------------------- */
+size_t lt_linear_backward_workspace_bytes(const lt_linear* lin, int64_t tokens, int32_t dtype);
+/* x [T, in], y [T, out], lowrank_hid [T, lowrank] (written when lin->lowrank > 0), all in `dtype` */
+int lt_linear_forward(const lt_linear* lin, int64_t tokens, int32_t dtype, const void* x, void* y, void* lowrank_hid,
+                      void* stream);
+/* dx may be NULL; dy [T, out]; lowrank_hid as written by lt_linear_forward */
+int lt_linear_backward(const lt_linear* lin, int64_t tokens, int32_t dtype, const void* x, const void* dy,
+                       const void* lowrank_hid, void* dx, const lt_linear_grads* grads, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/* ---- block-sparse matmul alone (weight in the native [in_features, A, block] format) ----------------------------------- */
+int lt_blocksparse_forward(const lt_linear* lin, int64_t tokens, int32_t dtype, const void* x, void* y, void* stream);
+/* dx and/or dweight may be NULL */
+int lt_blocksparse_backward(const lt_linear* lin, int64_t tokens, int32_t dtype, const void* x, const void* dy, void* dx,
+                            void* dweight, void* stream);
+
+/* ---- LayerNorm over the last dimension -------------------------------------------------------------------------------- */
+/* x [T, H] in x_dtype -> y [T, H] in y_dtype; stats [T, 2] = (mean, rstd) written when non-NULL */
+int lt_layernorm_forward(int64_t tokens, int32_t hidden, float eps, int32_t x_dtype, const void* x, const float* weight,
+                         const float* bias, int32_t y_dtype, void* y, float* stats, void* stream);
+size_t lt_layernorm_backward_workspace_bytes(int64_t tokens, int32_t hidden);
+/* dx = LN'(dy) [+ residual_grad]; dweight / dbias fp32 [H]; stats from the forward */
+int lt_layernorm_backward(int64_t tokens, int32_t hidden, int32_t x_dtype, const void* x, const float* stats,
+                          const float* weight, int32_t dy_dtype, const void* dy, int32_t dx_dtype,
+                          const void* residual_grad, void* dx, float* dweight, float* dbias, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* ---- activation alone (for tests of the in-register maths) ------------------------------------------------------------ */
+/* pre [T, 2I or I] -> hid [T, I] */
+int lt_activation_forward(int64_t tokens, int32_t intermediate, int32_t gated, int32_t act, int32_t dtype,
+                          const void* pre, void* hid, void* stream);
+/* d_hid [T, I], pre -> d_pre [T, 2I or I] */
+int lt_activation_backward(int64_t tokens, int32_t intermediate, int32_t gated, int32_t act, int32_t dtype,
+                           const void* pre, const void* d_hid, void* d_pre, void* stream);
+
+/* ---- dropout mask of a [T, H] output: keep[t*H + h] in {0,1}, the mask the fused kernels apply for (seed, offset) ------- */
+int lt_dropout_mask(int64_t tokens, int32_t hidden, float p, uint64_t seed, uint64_t offset, uint8_t* keep, void* stream);
+
+/* ---- plain GEMM on the library's kernels (tests and benchmarks of the MFMA core) -------------------------------------- */
+/* C[M,N] = op(A) op(B): a_kmajor != 0: A is [M,K] row-major, else [K,M]; b_kmajor != 0: B is [N,K] row-major, else [K,N].
+ * force_generic != 0 selects the any-shape kernel even when the tiled bf16 kernel applies. */
+int lt_gemm(int32_t dtype, int64_t m, int64_t n, int64_t k, const void* a, int32_t a_kmajor, const void* b,
+            int32_t b_kmajor, int32_t c_dtype, void* c, int32_t force_generic, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LEANFFN_H */

@@ -1,0 +1,50 @@
+"""Builds lean_transformer_amd/csrc/libleanffn.so from the HIP sources with hipcc for gfx950 (cross-compiles without a GPU).
+
+    python -m lean_transformer_amd._build
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(CSRC, "libleanffn.so")
+SOURCES = ["ffn.hip", "elementwise.hip", "gemm_generic.hip", "gemm_mfma_bf16.hip"]
+# -packed-fp32-ops is switched off: the compiler must not form v_pk_{add,mul,fma}_f32 from scalar float code
+FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + proc.stdout)
+    return proc.stdout
+
+
+def build(verbose: bool = False, extra_flags=()) -> str:
+    """Compile every translation unit (in parallel) and link the shared library; returns its path."""
+    hipcc = _hipcc()
+    objects = [os.path.join(CSRC, src.replace(".hip", ".o")) for src in SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        out = _run([hipcc, *FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
+        if verbose and out.strip():
+            print(out)
+
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        list(pool.map(compile_one, zip(SOURCES, objects)))
+    _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objects, "-o", LIB_PATH])
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

@@ -1,0 +1,157 @@
+"""ctypes binding of csrc/libleanffn.so (declarations: include/leanffn.h).
+
+The library is the only compute backend of this package: there is no fallback.  ``lib()`` raises if the shared object has
+not been built (``python -m lean_transformer_amd._build``), and every call raises ``RuntimeError`` with the library's own
+message when it returns a non-zero status.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_size_t, c_uint8, c_uint64, c_void_p
+from typing import Optional
+
+import torch
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libleanffn.so")
+
+LT_F32, LT_BF16 = 0, 1
+_DTYPES = {torch.float32: LT_F32, torch.bfloat16: LT_BF16}
+
+# every function include/leanffn.h declares; the not-gpu tests check that the built library exports all of them
+EXPORTED_SYMBOLS = (
+    "lt_version", "lt_last_error",
+    "lt_ffn_forward_workspace_bytes", "lt_ffn_backward_workspace_bytes", "lt_ffn_forward", "lt_ffn_backward",
+    "lt_linear_backward_workspace_bytes", "lt_linear_forward", "lt_linear_backward",
+    "lt_blocksparse_forward", "lt_blocksparse_backward",
+    "lt_layernorm_forward", "lt_layernorm_backward_workspace_bytes", "lt_layernorm_backward",
+    "lt_activation_forward", "lt_activation_backward", "lt_dropout_mask", "lt_gemm",
+)
+
+
+class LtLinear(ctypes.Structure):
+    _fields_ = [
+        ("weight", c_void_p), ("bias", c_void_p), ("lowrank_first", c_void_p), ("lowrank_second", c_void_p),
+        ("forward_indices", c_void_p), ("backward_indices", c_void_p),
+        ("in_features", c_int32), ("out_features", c_int32), ("lowrank", c_int32), ("block", c_int32),
+        ("blocks_per_out", c_int32), ("blocks_per_in", c_int32),
+    ]
+
+
+class LtLinearGrads(ctypes.Structure):
+    _fields_ = [("weight", c_void_p), ("bias", c_void_p), ("lowrank_first", c_void_p), ("lowrank_second", c_void_p)]
+
+
+class LtFfnDesc(ctypes.Structure):
+    _fields_ = [
+        ("tokens", c_int64), ("hidden", c_int32), ("intermediate", c_int32), ("gated", c_int32), ("act", c_int32),
+        ("residual", c_int32), ("io_dtype", c_int32), ("compute_dtype", c_int32), ("ln_eps", c_float),
+        ("dropout_p", c_float), ("dropout_seed", c_uint64), ("dropout_offset", c_uint64),
+        ("ln_weight", c_void_p), ("ln_bias", c_void_p), ("post_ln_weight", c_void_p), ("post_ln_bias", c_void_p),
+        ("i2h", LtLinear), ("h2o", LtLinear),
+    ]
+
+
+class LtFfnSaved(ctypes.Structure):
+    _fields_ = [("pre_activation", c_void_p), ("ln_stats", c_void_p), ("post_ln_input", c_void_p),
+                ("i2h_lowrank_hid", c_void_p), ("h2o_lowrank_hid", c_void_p)]
+
+
+class LtFfnGrads(ctypes.Structure):
+    _fields_ = [("dx", c_void_p), ("ln_weight", c_void_p), ("ln_bias", c_void_p), ("post_ln_weight", c_void_p),
+                ("post_ln_bias", c_void_p), ("i2h", LtLinearGrads), ("h2o", LtLinearGrads)]
+
+
+_lib = None
+
+
+def _declare(lib):
+    lib.lt_version.restype = c_char_p
+    lib.lt_last_error.restype = c_char_p
+    lib.lt_ffn_forward_workspace_bytes.restype = c_size_t
+    lib.lt_ffn_forward_workspace_bytes.argtypes = [POINTER(LtFfnDesc)]
+    lib.lt_ffn_backward_workspace_bytes.restype = c_size_t
+    lib.lt_ffn_backward_workspace_bytes.argtypes = [POINTER(LtFfnDesc)]
+    lib.lt_ffn_forward.argtypes = [POINTER(LtFfnDesc), c_void_p, c_void_p, POINTER(LtFfnSaved), c_void_p, c_size_t, c_void_p]
+    lib.lt_ffn_backward.argtypes = [POINTER(LtFfnDesc), c_void_p, c_void_p, POINTER(LtFfnSaved), POINTER(LtFfnGrads),
+                                    c_void_p, c_size_t, c_void_p]
+    lib.lt_linear_backward_workspace_bytes.restype = c_size_t
+    lib.lt_linear_backward_workspace_bytes.argtypes = [POINTER(LtLinear), c_int64, c_int32]
+    lib.lt_linear_forward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.lt_linear_backward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       POINTER(LtLinearGrads), c_void_p, c_size_t, c_void_p]
+    lib.lt_blocksparse_forward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p]
+    lib.lt_blocksparse_backward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p]
+    lib.lt_layernorm_forward.argtypes = [c_int64, c_int32, c_float, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
+                                         c_void_p, c_void_p, c_void_p]
+    lib.lt_layernorm_backward_workspace_bytes.restype = c_size_t
+    lib.lt_layernorm_backward_workspace_bytes.argtypes = [c_int64, c_int32]
+    lib.lt_layernorm_backward.argtypes = [c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p,
+                                          c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
+    lib.lt_activation_forward.argtypes = [c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p]
+    lib.lt_activation_backward.argtypes = [c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+                                           c_void_p]
+    lib.lt_dropout_mask.argtypes = [c_int64, c_int32, c_float, c_uint64, c_uint64, c_void_p, c_void_p]
+    lib.lt_gemm.argtypes = [c_int32, c_int64, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p,
+                            c_int32, c_void_p]
+    for name in EXPORTED_SYMBOLS:
+        fn = getattr(lib, name)
+        if fn.restype is ctypes.c_int:  # default restype: these return lt_status
+            fn.restype = c_int32
+
+
+def lib():
+    """The loaded library; raises if it was never built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP kernels of lean_transformer_amd are not built. "
+                "Run `python -m lean_transformer_amd._build` (needs hipcc; cross-compiles for gfx950 without a GPU).")
+        loaded = ctypes.CDLL(LIB_PATH)
+        _declare(loaded)
+        _lib = loaded
+    return _lib
+
+
+def check(status: int, what: str):
+    if status != 0:
+        message = lib().lt_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed (lt_status {status}): {message}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError(f"the HIP kernels take float32 and bfloat16 tensors, not {dtype}") from None
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    """device address of a tensor (None -> NULL)"""
+    return None if t is None else t.data_ptr()
+
+
+def require_gpu(*tensors: Optional[torch.Tensor]):
+    """All tensors must live on one GPU; there is no CPU implementation behind this package."""
+    device = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                f"lean_transformer_amd runs on AMD GPUs only (got a tensor on {t.device}); its HIP kernels have no CPU "
+                "counterpart. Move the module and its inputs to the GPU.")
+        if device is None:
+            device = t.device
+        elif t.device != device:
+            raise RuntimeError(f"tensors on different devices: {device} and {t.device}")
+    return device
+
+
+def current_stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    """scratch memory from PyTorch's caching allocator (256-byte aligned like every fresh block of it)"""
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)

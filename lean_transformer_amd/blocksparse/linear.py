@@ -1,0 +1,224 @@
+"""Weight containers and the "generalized linear" layer: (dense | block-sparse) main matrix + optional low-rank term,
+shareable between layers, with a per-layer low-rank adapter.
+
+Same classes, constructor arguments, attributes and state_dict keys as lean_transformer/blocksparse/linear.py:19-149, so a
+checkpoint of the reference loads unchanged.  The forward / backward of ``_GeneralizedLinear`` run on the HIP kernels
+(lt_linear_forward / lt_linear_backward) instead of F.linear / addmm / the embedding_bag-based sparse matmul.
+"""
+import math
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from .. import _native as nat
+from .layout import get_blocksparse_layout, get_indices_from_layout
+
+
+class GeneralizedMatrix(nn.Module):
+    """A module that stores a shared pytorch tensor for use in GeneralizedLinear layers"""
+
+    def __init__(self, in_features: int, out_features: int, blocksparse_layout: Optional[str] = None,
+                 lowrank_dim: int = 0, blocksparse_backend: str = 'native'):
+        super().__init__()
+        self.out_features, self.in_features = out_features, in_features
+        if blocksparse_backend != 'native':
+            raise NotImplementedError(
+                f"blocksparse_backend={blocksparse_backend!r}: only the 'native' weight format is implemented "
+                "(its matmul runs on HIP kernels; there is no Triton path)")
+        self.blocksparse_backend = blocksparse_backend
+
+        if blocksparse_layout is None:
+            # fully-connected weight matrix
+            self.weight = nn.Parameter(torch.empty(out_features, in_features))
+            nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+            self.layout = self.forward_indices = self.backward_indices = None
+        else:
+            layout = get_blocksparse_layout(out_features, in_features, blocksparse_layout)
+            assert out_features / layout.shape[0] == in_features / layout.shape[1] == in_features // layout.shape[1]
+            block_size = in_features // layout.shape[1]
+            self.register_buffer("layout", layout, persistent=True)
+            forward_indices, backward_indices = get_indices_from_layout(layout)
+            self.register_buffer("forward_indices", forward_indices, persistent=True)
+            self.register_buffer("backward_indices", backward_indices, persistent=True)
+            active_blocks_per_input = self.forward_indices.numel() // (in_features // block_size)
+            self.weight = nn.Parameter(torch.empty(in_features, active_blocks_per_input, block_size))
+            torch.nn.init.normal_(self.weight, std=math.sqrt(2.0 / (5 * min(out_features, in_features))))
+
+        if lowrank_dim:
+            self.lowrank_first = nn.Parameter(torch.zeros(lowrank_dim, self.in_features))
+            self.lowrank_second = nn.Parameter(torch.zeros(self.out_features, lowrank_dim))
+            nn.init.normal_(self.lowrank_first, std=math.sqrt(2.0 / (5 * min(out_features, in_features))))
+            nn.init.normal_(self.lowrank_second, std=math.sqrt(2.0 / (5 * min(out_features, in_features))))
+        else:
+            self.lowrank_first = self.lowrank_second = None
+
+    @property
+    def shape(self):
+        return self.out_features, self.in_features
+
+    @property
+    def matmul_op(self):
+        """The reference's slot for a Triton matmul object; always None here (the 'native' format is the only one)."""
+        return None
+
+    def __repr__(self):
+        return f"{self.__class__.__name__}{tuple(self.shape)}"
+
+    def forward(self, input: torch.Tensor, *, ignore_lowrank: bool = False):
+        """
+        Multiply input tensor by this matrix with the same semantics as in torch.nn.Linear(..., bias=False)
+
+        :param ignore_lowrank: if True, the low-rank components (lowrank_dim) will not be used in matrix multiplication
+        """
+        use_lowrank = self.lowrank_first is not None and not ignore_lowrank
+        return _GeneralizedLinear.apply(
+            input, self.weight, None, self.lowrank_first if use_lowrank else None,
+            self.lowrank_second if use_lowrank else None, self.forward_indices, self.backward_indices, None)
+
+
+class GeneralizedLinear(nn.Linear):
+    """A linear layer with a shared full-rank matrix and an individual low-rank adapter"""
+
+    def __init__(self, matrix: GeneralizedMatrix, adapter_dim: int = 0, bias: bool = True):
+        nn.Module.__init__(self)
+        self.matrix = matrix
+        self.out_features, self.in_features = self.matrix.shape
+        self.bias = nn.Parameter(torch.zeros(self.out_features)) if bias else None
+
+        if adapter_dim != 0:
+            self.adapter_first = nn.Parameter(torch.zeros(adapter_dim, self.in_features))
+            self.adapter_second = nn.Parameter(torch.zeros(self.out_features, adapter_dim))
+            # initialize in accordance with https://arxiv.org/pdf/2106.09685.pdf
+            nn.init.xavier_normal_(self.adapter_first)
+            nn.init.zeros_(self.adapter_second)
+        else:
+            self.adapter_first = self.adapter_second = None
+
+    def get_combined_lowrank_components(self) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        """Group together low-rank matrices from this layer's adapter and GeneralizedMatrix for faster matmul"""
+        if self.adapter_first is not None and self.matrix.lowrank_first is None:
+            return self.adapter_first, self.adapter_second
+        elif self.adapter_first is None and self.matrix.lowrank_first is not None:
+            return self.matrix.lowrank_first, self.matrix.lowrank_second
+        elif self.adapter_first is not None and self.matrix.lowrank_first is not None:
+            combined_first = torch.cat([self.matrix.lowrank_first, self.adapter_first], dim=0)
+            combined_second = torch.cat([self.matrix.lowrank_second, self.adapter_second], dim=1)
+            return combined_first, combined_second
+        else:
+            return None, None
+
+    @property
+    def weight(self):
+        return self.matrix.weight
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        return _GeneralizedLinear.apply(
+            input, self.weight, self.bias, *self.get_combined_lowrank_components(),
+            self.matrix.forward_indices, self.matrix.backward_indices, self.matrix.matmul_op)
+
+
+def compute_dtype_for(weight: torch.Tensor) -> torch.dtype:
+    """dtype of GEMM operands: the autocast dtype when autocast is on (as F.linear would use), else the weight's dtype"""
+    if torch.is_autocast_enabled("cuda"):
+        dtype = torch.get_autocast_dtype("cuda")
+        if dtype != torch.bfloat16:
+            raise NotImplementedError(f"autocast to {dtype}: the HIP kernels compute in bfloat16 or float32")
+        return dtype
+    return weight.dtype
+
+
+def _as(t: Optional[torch.Tensor], dtype: torch.dtype) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    t = t.detach()
+    if t.dtype != dtype:
+        t = t.to(dtype)
+    return t.contiguous()
+
+
+def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices, backward_indices) -> "nat.LtLinear":
+    """ctypes descriptor of one projection; all tensors already in their final dtype and contiguous"""
+    desc = nat.LtLinear()
+    desc.weight = nat.ptr(weight)
+    desc.bias = nat.ptr(bias_f32)
+    desc.lowrank_first, desc.lowrank_second = nat.ptr(lowrank_first), nat.ptr(lowrank_second)
+    desc.lowrank = 0 if lowrank_first is None else lowrank_first.shape[0]
+    if forward_indices is None:
+        desc.out_features, desc.in_features = weight.shape
+        desc.block = desc.blocks_per_in = desc.blocks_per_out = 0
+    else:
+        in_features, blocks_per_in, block = weight.shape
+        desc.in_features, desc.out_features = in_features, forward_indices.shape[0] * block
+        desc.block, desc.blocks_per_in, desc.blocks_per_out = block, blocks_per_in, forward_indices.shape[1]
+        desc.forward_indices, desc.backward_indices = nat.ptr(forward_indices), nat.ptr(backward_indices)
+    return desc
+
+
+class _GeneralizedLinear(torch.autograd.Function):
+    """y = x W^T (+ bias) (+ (x L1^T) L2^T) with W dense or block-sparse.  Argument order as in the reference's
+    _GeneralizedLinear.apply (linear.py:147-149): input, main_weight, bias, lowrank_first, lowrank_second,
+    forward_indices, backward_indices[, matmul_op]."""
+
+    @staticmethod
+    def forward(ctx, *args):
+        ctx._nargs = len(args)
+        (input, main_weight, bias, lowrank_first, lowrank_second, forward_indices, backward_indices,
+         matmul_op) = tuple(args) + (None,) * (8 - len(args))
+        if matmul_op is not None:
+            raise NotImplementedError("matmul_op plug-ins (Triton) are not supported; the block-sparse matmul is built in")
+        device = nat.require_gpu(input, main_weight, bias, lowrank_first, lowrank_second, forward_indices, backward_indices)
+        dtype = compute_dtype_for(main_weight)
+        x = _as(input, dtype).reshape(-1, input.shape[-1])
+        w = _as(main_weight, dtype)
+        l1, l2 = _as(lowrank_first, dtype), _as(lowrank_second, dtype)
+        b32 = _as(bias, torch.float32)
+        fwd = None if forward_indices is None else forward_indices.to(torch.int32).contiguous()
+        bwd = None if backward_indices is None else backward_indices.to(torch.int64).contiguous()
+        desc = linear_desc(w, b32, l1, l2, fwd, bwd)
+        if x.shape[1] != desc.in_features:
+            raise ValueError(f"input has {x.shape[1]} features, the weight takes {desc.in_features}")
+        tokens = x.shape[0]
+        y = torch.empty(tokens, desc.out_features, dtype=dtype, device=device)
+        hid = torch.empty(tokens, desc.lowrank, dtype=dtype, device=device) if desc.lowrank else None
+        if tokens > 0:
+            nat.check(nat.lib().lt_linear_forward(desc, tokens, nat.dtype_code(dtype), nat.ptr(x), nat.ptr(y), nat.ptr(hid),
+                                                  nat.current_stream(device)), "lt_linear_forward")
+        ctx.save_for_backward(input, hid, main_weight, lowrank_first, lowrank_second, forward_indices, backward_indices)
+        ctx._dtype, ctx._has_bias = dtype, bias is not None
+        return y.view(*input.shape[:-1], desc.out_features)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, hid, main_weight, lowrank_first, lowrank_second, forward_indices, backward_indices = ctx.saved_tensors
+        dtype = ctx._dtype
+        device = grad_output.device
+        need = tuple(ctx.needs_input_grad) + (False,) * 8
+        x = _as(input, dtype).reshape(-1, input.shape[-1])
+        dy = _as(grad_output, dtype).reshape(x.shape[0], -1)
+        w = _as(main_weight, dtype)
+        l1, l2 = _as(lowrank_first, dtype), _as(lowrank_second, dtype)
+        fwd = None if forward_indices is None else forward_indices.to(torch.int32).contiguous()
+        bwd = None if backward_indices is None else backward_indices.to(torch.int64).contiguous()
+        desc = linear_desc(w, None, l1, l2, fwd, bwd)
+        tokens = x.shape[0]
+        grads = nat.LtLinearGrads()
+        dx = torch.empty_like(x) if need[0] else None
+        dw = torch.empty_like(w) if need[1] else None
+        db = torch.empty(desc.out_features, dtype=torch.float32, device=device) if (ctx._has_bias and need[2]) else None
+        dl1 = torch.empty_like(l1) if (l1 is not None and need[3]) else None
+        dl2 = torch.empty_like(l2) if (l2 is not None and need[4]) else None
+        grads.weight, grads.bias, grads.lowrank_first, grads.lowrank_second = (nat.ptr(dw), nat.ptr(db), nat.ptr(dl1),
+                                                                               nat.ptr(dl2))
+        if tokens > 0:
+            lib = nat.lib()
+            ws = nat.workspace(lib.lt_linear_backward_workspace_bytes(desc, tokens, nat.dtype_code(dtype)), device)
+            nat.check(lib.lt_linear_backward(desc, tokens, nat.dtype_code(dtype), nat.ptr(x), nat.ptr(dy), nat.ptr(hid),
+                                             nat.ptr(dx), grads, nat.ptr(ws), ws.numel(), nat.current_stream(device)),
+                      "lt_linear_backward")
+        else:
+            for g in (dw, db, dl1, dl2):
+                if g is not None:
+                    g.zero_()
+        out = (None if dx is None else dx.view(input.shape), dw, db, dl1, dl2, None, None, None)
+        return out[:ctx._nargs]  # callers pass 2..8 positional arguments (everything after main_weight is optional)

@@ -1,0 +1,77 @@
+"""Block-sparse matmul in the reference's "native" weight format, on the HIP kernels.
+
+Same functions and argument meaning as lean_transformer/blocksparse/native_backend.py:9-76; the reference's per-block batched
+matmul + embedding_bag / embedding gather is replaced by one kernel launch that walks the index tables.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _native as nat
+
+
+def _sparse_desc(weight: torch.Tensor, forward_indices: Optional[torch.Tensor], backward_indices: Optional[torch.Tensor],
+                 out_features: int) -> "nat.LtLinear":
+    in_features, blocks_per_in, block = weight.shape
+    desc = nat.LtLinear()
+    desc.weight = nat.ptr(weight)
+    desc.in_features, desc.out_features = in_features, out_features
+    desc.block, desc.blocks_per_in = block, blocks_per_in
+    desc.blocks_per_out = (in_features // block) * blocks_per_in // (out_features // block)
+    # the kernels read whichever table their direction needs; the other one may be absent when this is called directly
+    desc.forward_indices = nat.ptr(forward_indices) if forward_indices is not None else nat.ptr(backward_indices)
+    desc.backward_indices = nat.ptr(backward_indices) if backward_indices is not None else nat.ptr(forward_indices)
+    return desc
+
+
+def blocksparse_matmul(input: torch.Tensor, weight: torch.Tensor, forward_indices: torch.Tensor) -> torch.Tensor:
+    """
+    :param input: tensor [*batch_dims, in_features]
+    :param weight: tensor [in_features, active_blocks_per_input, block_size]
+    :param forward_indices: the first output of get_indices_from_layout(...), int32 [num_output_blocks, K]
+    :returns: tensor [*batch_dims, out_features]
+    """
+    assert input.shape[-1] == weight.shape[0]
+    device = nat.require_gpu(input, weight, forward_indices)
+    block = weight.shape[2]
+    out_features = forward_indices.shape[0] * block
+    x = input.reshape(-1, input.shape[-1]).contiguous()
+    w = weight.contiguous()
+    if w.dtype != x.dtype:
+        w = w.to(x.dtype)
+    fwd = forward_indices.to(torch.int32).contiguous()
+    y = torch.empty(x.shape[0], out_features, dtype=x.dtype, device=device)
+    if x.shape[0] > 0:
+        desc = _sparse_desc(w, fwd, None, out_features)
+        nat.check(nat.lib().lt_blocksparse_forward(desc, x.shape[0], nat.dtype_code(x.dtype), nat.ptr(x), nat.ptr(y),
+                                                    nat.current_stream(device)), "lt_blocksparse_forward")
+    return y.view(*input.shape[:-1], out_features)
+
+
+def blocksparse_matmul_backward(grad_output: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
+                                backward_indices: torch.Tensor, input_requires_grad: bool = True,
+                                weight_requires_grad: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Gradients of blocksparse_matmul w.r.t. input and/or weight; a gradient that is not requested comes back empty."""
+    assert input_requires_grad or weight_requires_grad, "computing backward but none of the inputs requires grad"
+    device = nat.require_gpu(grad_output, input, weight, backward_indices)
+    x = input.reshape(-1, input.shape[-1]).contiguous()
+    dy = grad_output.reshape(x.shape[0], -1).contiguous()
+    if dy.dtype != x.dtype:
+        dy = dy.to(x.dtype)
+    w = weight.contiguous()
+    if w.dtype != x.dtype:
+        w = w.to(x.dtype)
+    bwd = backward_indices.to(torch.int64).contiguous()
+    grad_input = torch.empty_like(x) if input_requires_grad else None
+    grad_weight = torch.empty_like(w) if weight_requires_grad else None
+    if x.shape[0] > 0:
+        desc = _sparse_desc(w, None, bwd, dy.shape[1])
+        nat.check(nat.lib().lt_blocksparse_backward(desc, x.shape[0], nat.dtype_code(x.dtype), nat.ptr(x), nat.ptr(dy),
+                                                     nat.ptr(grad_input), nat.ptr(grad_weight),
+                                                     nat.current_stream(device)), "lt_blocksparse_backward")
+    else:
+        if grad_weight is not None:
+            grad_weight.zero_()
+    empty = torch.empty(0, device=device, dtype=x.dtype)
+    return (grad_input.view(*grad_output.shape[:-1], input.shape[-1]) if grad_input is not None else empty,
+            grad_weight.to(weight.dtype) if grad_weight is not None else empty)

@@ -1,0 +1,415 @@
+// HBM-bound kernels of the FFN path: LayerNorm forward / backward with wavefront-shuffle row reductions, column sums for
+// bias / LayerNorm-parameter gradients, stand-alone activation forward / backward, dropout replay and the dropout mask.
+#include "lt_internal.h"
+
+namespace {
+
+constexpr int LN_MAXV = 32;  // float4 per lane held in registers: rows up to 64 * 4 * 32 = 8192 elements stay on chip
+
+// ---------------------------------------------------------------------------------------------------------------------
+// LayerNorm forward: one wavefront per row.  The row is read once into registers (when hidden % 4 == 0 and it fits), the
+// mean and the centred second moment are reduced across the 64 lanes with shuffles, and the normalised row is written in
+// the GEMM operand dtype.  TAIL fuses what follows a post-LayerNorm: dropout, then the residual add.
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename TX, typename TY, typename TR, bool TAIL>
+__global__ __launch_bounds__(256) void ln_fwd_kernel(int64_t T, int H, float eps, const TX* __restrict__ x,
+                                                      const float* __restrict__ w, const float* __restrict__ b,
+                                                      TY* __restrict__ y, float* __restrict__ stats,
+                                                      const TR* __restrict__ residual, DropoutParams drop, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= T) return;
+  const TX* xr = x + row * H;
+  const float inv_h = 1.0f / (float)H;
+  float mean, rstd;
+  if (vec) {
+    float v[LN_MAXV][4];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_MAXV; i++) {
+      const int c = (i * 64 + lane) * 4;
+      if (c < H) {
+        load4(xr + c, v[i]);
+        s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+      }
+    }
+    mean = wave_sum(s) * inv_h;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_MAXV; i++) {
+      const int c = (i * 64 + lane) * 4;
+      if (c < H) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float d = v[i][e] - mean;
+          q += d * d;
+        }
+      }
+    }
+    rstd = 1.0f / sqrtf(wave_sum(q) * inv_h + eps);
+    if (y) {
+#pragma unroll
+      for (int i = 0; i < LN_MAXV; i++) {
+        const int c = (i * 64 + lane) * 4;
+        if (c < H) {
+          float wv[4], bv[4], o[4];
+          load4(w + c, wv);
+          load4(b + c, bv);
+#pragma unroll
+          for (int e = 0; e < 4; e++) o[e] = (v[i][e] - mean) * rstd * wv[e] + bv[e];
+          if constexpr (TAIL) {
+            if (drop.p > 0.f) {
+              bool keep[4];
+              dropout_keep4(drop, row * H + c, keep);
+#pragma unroll
+              for (int e = 0; e < 4; e++) o[e] = keep[e] ? o[e] * drop.scale : 0.f;
+            }
+            if (residual) {
+              float rv[4];
+              load4(residual + row * H + c, rv);
+#pragma unroll
+              for (int e = 0; e < 4; e++) o[e] += rv[e];
+            }
+          }
+          store4(y + row * H + c, o);
+        }
+      }
+    }
+  } else {
+    float s = 0.f;
+    for (int c = lane; c < H; c += 64) s += ldf(xr, c);
+    mean = wave_sum(s) * inv_h;
+    float q = 0.f;
+    for (int c = lane; c < H; c += 64) {
+      const float d = ldf(xr, c) - mean;
+      q += d * d;
+    }
+    rstd = 1.0f / sqrtf(wave_sum(q) * inv_h + eps);
+    if (y) {
+      for (int c = lane; c < H; c += 64) {
+        float o = (ldf(xr, c) - mean) * rstd * w[c] + b[c];
+        if constexpr (TAIL) {
+          if (drop.p > 0.f) o = dropout_keep(drop, row * H + c) ? o * drop.scale : 0.f;
+          if (residual) o += ldf(residual, row * H + c);
+        }
+        stf(y, row * H + c, o);
+      }
+    }
+  }
+  if (stats && lane == 0) {
+    stats[row * 2] = mean;
+    stats[row * 2 + 1] = rstd;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// LayerNorm backward.  A workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ...; its 256 threads split the columns.
+//   dxhat = dy * w;  c1 = mean(dxhat);  c2 = mean(dxhat * xhat);  dx = rstd * (dxhat - c1 - xhat * c2) [+ residual grad]
+// Column sums of dy * xhat (-> dweight) and dy (-> dbias) are kept per thread across the rows of the workgroup and written
+// as one partial row per workgroup; lt_colreduce sums the partial rows.
+// ---------------------------------------------------------------------------------------------------------------------
+constexpr int LNB_MAXC = 32;  // columns per thread (hidden <= 256 * 32 = 8192) for the register-resident partial sums
+
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();  // protect `red` against the previous use
+  if (lane == 0) {
+    red[wave * 2] = a;
+    red[wave * 2 + 1] = b;
+  }
+  __syncthreads();
+  a = red[0] + red[2] + red[4] + red[6];
+  b = red[1] + red[3] + red[5] + red[7];
+}
+
+template <typename TX, typename TDY, typename TDX>
+__global__ __launch_bounds__(256) void ln_bwd_kernel(int64_t T, int H, const TX* __restrict__ x,
+                                                      const float* __restrict__ stats, const float* __restrict__ w,
+                                                      const TDY* __restrict__ dy, const TDX* __restrict__ residual_grad,
+                                                      TDX* __restrict__ dx, float* __restrict__ partial) {
+  __shared__ float red[8];
+  const int tid = threadIdx.x;
+  float pw[LNB_MAXC], pb[LNB_MAXC];
+#pragma unroll
+  for (int i = 0; i < LNB_MAXC; i++) pw[i] = pb[i] = 0.f;
+  const float inv_h = 1.0f / (float)H;
+  for (int64_t row = blockIdx.x; row < T; row += gridDim.x) {
+    const float mean = stats[row * 2], rstd = stats[row * 2 + 1];
+    const TX* xr = x + row * H;
+    const TDY* dyr = dy + row * H;
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < LNB_MAXC; i++) {
+      const int c = tid + i * 256;
+      if (c < H) {
+        const float xh = (ldf(xr, c) - mean) * rstd, g = ldf(dyr, c);
+        const float dxh = g * w[c];
+        s1 += dxh;
+        s2 += dxh * xh;
+        pw[i] += g * xh;
+        pb[i] += g;
+      }
+    }
+    block_sum2(s1, s2, red);
+    const float c1 = s1 * inv_h, c2 = s2 * inv_h;
+    if (dx) {
+#pragma unroll
+      for (int i = 0; i < LNB_MAXC; i++) {
+        const int c = tid + i * 256;
+        if (c < H) {
+          const float xh = (ldf(xr, c) - mean) * rstd;
+          float v = rstd * (ldf(dyr, c) * w[c] - c1 - xh * c2);
+          if (residual_grad) v += ldf(residual_grad, row * H + c);
+          stf(dx, row * H + c, v);
+        }
+      }
+    }
+  }
+  if (partial) {
+#pragma unroll
+    for (int i = 0; i < LNB_MAXC; i++) {
+      const int c = tid + i * 256;
+      if (c < H) {
+        partial[((int64_t)blockIdx.x * 2) * H + c] = pw[i];
+        partial[((int64_t)blockIdx.x * 2 + 1) * H + c] = pb[i];
+      }
+    }
+  }
+}
+
+// out[c] = sum_r partial[r * stride + c], one thread per column (rows are few)
+__global__ void colreduce_kernel(int rows, int64_t stride, int cols, const float* __restrict__ partial,
+                                 float* __restrict__ out) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  float s = 0.f;
+  for (int r = 0; r < rows; r++) s += partial[(int64_t)r * stride + c];
+  out[c] = s;
+}
+
+// partial[blockIdx.y][c] = sum over this row-slice of in[t, c]; 64 column lanes x 4 row lanes per workgroup
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(int64_t rows, int cols, int64_t ld, const T* __restrict__ in,
+                                                              int64_t rows_per_slice, float* __restrict__ partial) {
+  __shared__ float red[4][64];
+  const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + cl;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice, r1 = min(rows, r0 + rows_per_slice);
+  float s = 0.f;
+  if (c < cols)
+    for (int64_t r = r0 + rl; r < r1; r += 4) s += ldf(in, r * ld + c);
+  red[rl][cl] = s;
+  __syncthreads();
+  if (rl == 0 && c < cols) partial[(int64_t)blockIdx.y * cols + c] = red[0][cl] + red[1][cl] + red[2][cl] + red[3][cl];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// stand-alone (gated) activation forward / backward on a saved pre-activation
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename TC>
+__global__ void act_fwd_kernel(int64_t T, int64_t I, int gated, int act, const TC* __restrict__ pre, TC* __restrict__ hid) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * I) return;
+  const int64_t t = idx / I, i = idx % I;
+  const int64_t ldp = gated ? 2 * I : I;
+  float a = act_value<PRECISE>(act, ldf(pre, t * ldp + i));
+  if (gated) a *= ldf(pre, t * ldp + I + i);
+  stf(hid, idx, a);
+}
+
+template <typename TC>
+__global__ void act_bwd_kernel(int64_t T, int64_t I, int gated, int act, const TC* __restrict__ pre,
+                               const TC* __restrict__ dhid, TC* __restrict__ dpre) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * I) return;
+  const int64_t t = idx / I, i = idx % I;
+  const int64_t ldp = gated ? 2 * I : I;
+  float a, da;
+  act_eval<PRECISE>(act, ldf(pre, t * ldp + i), a, da);
+  const float dh = ldf(dhid, idx);
+  if (gated) {
+    const float pl = ldf(pre, t * ldp + I + i);
+    stf(dpre, t * ldp + i, dh * pl * da);
+    stf(dpre, t * ldp + I + i, dh * a);
+  } else {
+    stf(dpre, t * ldp + i, dh * da);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// dropout replay on the incoming gradient (and conversion to the GEMM operand dtype); mask bytes for tests
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void dropout_cast_kernel(int64_t n, const TI* __restrict__ in, TO* __restrict__ out, DropoutParams drop) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  float v = ldf(in, idx);
+  if (drop.p > 0.f) v = dropout_keep(drop, idx) ? v * drop.scale : 0.f;
+  stf(out, idx, v);
+}
+
+__global__ void dropout_mask_kernel(int64_t n, uint8_t* __restrict__ keep, DropoutParams drop) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  keep[idx] = drop.p > 0.f ? (dropout_keep(drop, idx) ? 1 : 0) : 1;
+}
+
+inline unsigned blocks_for(int64_t n, int threads) { return (unsigned)((n + threads - 1) / threads); }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------------------------
+// host-side launchers
+// ---------------------------------------------------------------------------------------------------------------------
+int lt_ln_forward(int64_t T, int H, float eps, int x_dtype, const void* x, const float* w, const float* b, int y_dtype,
+                  void* y, float* stats, int res_dtype, const void* residual, const DropoutParams* drop, bool tail,
+                  hipStream_t stream) {
+  LT_REQUIRE(T > 0 && H > 0 && x, LT_ERR_BAD_ARG, "layernorm: bad arguments");
+  LT_REQUIRE(!y || (w && b), LT_ERR_BAD_ARG, "layernorm: weight and bias are required when an output is requested");
+  // rows are held in registers and moved 4 elements at a time when the size and every pointer allow it
+  const int vec = (H & 3) == 0 && H <= 64 * 4 * LN_MAXV && lt_aligned(x, 16) && (!y || lt_aligned(y, 16)) &&
+                  (!w || lt_aligned(w, 16)) && (!b || lt_aligned(b, 16)) && (!residual || lt_aligned(residual, 16));
+  dim3 grid(blocks_for(T, 4)), block(256);
+  DropoutParams d = drop ? *drop : make_dropout(0.f, 0, 0);
+#define LT_LN_LAUNCH(TX, TY, TR, TAILV)                                                                              \
+  hipLaunchKernelGGL((ln_fwd_kernel<TX, TY, TR, TAILV>), grid, block, 0, stream, T, H, eps, (const TX*)x, w, b, (TY*)y, \
+                     stats, (const TR*)residual, d, vec)
+  if (!tail) {
+    if (x_dtype == LT_F32 && y_dtype == LT_F32) LT_LN_LAUNCH(float, float, float, false);
+    else if (x_dtype == LT_F32) LT_LN_LAUNCH(float, bf16, float, false);
+    else if (y_dtype == LT_F32) LT_LN_LAUNCH(bf16, float, float, false);
+    else LT_LN_LAUNCH(bf16, bf16, float, false);
+  } else {
+    // post-LayerNorm tail: input in the compute dtype, output and residual in the io dtype (res_dtype == y_dtype)
+    LT_REQUIRE(res_dtype == y_dtype, LT_ERR_BAD_ARG, "layernorm tail: residual and output dtypes differ");
+    if (x_dtype == LT_F32 && y_dtype == LT_F32) LT_LN_LAUNCH(float, float, float, true);
+    else if (x_dtype == LT_F32) LT_LN_LAUNCH(float, bf16, bf16, true);
+    else if (y_dtype == LT_F32) LT_LN_LAUNCH(bf16, float, float, true);
+    else LT_LN_LAUNCH(bf16, bf16, bf16, true);
+  }
+#undef LT_LN_LAUNCH
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+static int ln_bwd_blocks(int64_t T) { return (int)(T < 1024 ? T : 1024); }
+
+size_t lt_ln_backward_workspace(int64_t T, int H) { return (size_t)ln_bwd_blocks(T) * 2 * (size_t)H * sizeof(float); }
+
+int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* stats, const float* w, int dy_dtype,
+                   const void* dy, int dx_dtype, const void* residual_grad, void* dx, float* dweight, float* dbias,
+                   void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  LT_REQUIRE(T > 0 && H > 0 && x && stats && w && dy, LT_ERR_BAD_ARG, "layernorm backward: bad arguments");
+  LT_REQUIRE(H <= 256 * LNB_MAXC, LT_ERR_UNSUPPORTED, "layernorm backward: hidden size %d above %d", H, 256 * LNB_MAXC);
+  LT_REQUIRE((dweight == nullptr) == (dbias == nullptr), LT_ERR_BAD_ARG, "layernorm backward: pass both dweight and dbias or neither");
+  const int nb = ln_bwd_blocks(T);
+  float* partial = nullptr;
+  if (dweight) {
+    LT_REQUIRE(workspace && workspace_bytes >= lt_ln_backward_workspace(T, H), LT_ERR_WORKSPACE,
+               "layernorm backward: workspace of %zu bytes needed", lt_ln_backward_workspace(T, H));
+    partial = (float*)workspace;
+  }
+  dim3 grid(nb), block(256);
+#define LT_LNB_LAUNCH(TX, TDY, TDX)                                                                                      \
+  hipLaunchKernelGGL((ln_bwd_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
+                     (const TDX*)residual_grad, (TDX*)dx, partial)
+  const int key = (x_dtype == LT_BF16) * 4 + (dy_dtype == LT_BF16) * 2 + (dx_dtype == LT_BF16);
+  switch (key) {
+    case 0: LT_LNB_LAUNCH(float, float, float); break;
+    case 1: LT_LNB_LAUNCH(float, float, bf16); break;
+    case 2: LT_LNB_LAUNCH(float, bf16, float); break;
+    case 3: LT_LNB_LAUNCH(float, bf16, bf16); break;
+    case 4: LT_LNB_LAUNCH(bf16, float, float); break;
+    case 5: LT_LNB_LAUNCH(bf16, float, bf16); break;
+    case 6: LT_LNB_LAUNCH(bf16, bf16, float); break;
+    default: LT_LNB_LAUNCH(bf16, bf16, bf16); break;
+  }
+#undef LT_LNB_LAUNCH
+  LT_LAUNCH_CHECK();
+  if (dweight) {
+    // partial rows alternate (dweight, dbias): stride 2 * H between workgroups
+    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, nb, (int64_t)2 * H, H, partial,
+                       dweight);
+    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, nb, (int64_t)2 * H, H,
+                       partial + H, dbias);
+    LT_LAUNCH_CHECK();
+  }
+  return LT_OK;
+}
+
+static int colsum_slices(int64_t rows) {
+  int64_t s = (rows + 255) / 256;
+  return (int)(s < 1 ? 1 : (s > 64 ? 64 : s));
+}
+
+size_t lt_colsum_workspace(int64_t rows, int cols) { return (size_t)colsum_slices(rows) * (size_t)cols * sizeof(float); }
+
+int lt_colsum(int64_t rows, int cols, int64_t ld, int dtype, const void* in, float* out, void* workspace,
+              size_t workspace_bytes, hipStream_t stream) {
+  LT_REQUIRE(rows > 0 && cols > 0 && in && out, LT_ERR_BAD_ARG, "colsum: bad arguments");
+  LT_REQUIRE(workspace && workspace_bytes >= lt_colsum_workspace(rows, cols), LT_ERR_WORKSPACE,
+             "colsum: workspace of %zu bytes needed", lt_colsum_workspace(rows, cols));
+  const int slices = colsum_slices(rows);
+  const int64_t rps = (rows + slices - 1) / slices;
+  dim3 grid(blocks_for(cols, 64), slices), block(256);
+  float* partial = (float*)workspace;
+  if (dtype == LT_F32)
+    hipLaunchKernelGGL((colsum_partial_kernel<float>), grid, block, 0, stream, rows, cols, ld, (const float*)in, rps, partial);
+  else
+    hipLaunchKernelGGL((colsum_partial_kernel<bf16>), grid, block, 0, stream, rows, cols, ld, (const bf16*)in, rps, partial);
+  hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(cols, 256)), dim3(256), 0, stream, slices, (int64_t)cols, cols,
+                     partial, out);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+int lt_act_forward(int64_t T, int64_t I, int gated, int act, int dtype, const void* pre, void* hid, hipStream_t stream) {
+  LT_REQUIRE(T > 0 && I > 0 && pre && hid, LT_ERR_BAD_ARG, "activation: bad arguments");
+  dim3 grid(blocks_for(T * I, 256)), block(256);
+  if (dtype == LT_F32)
+    hipLaunchKernelGGL((act_fwd_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre, (float*)hid);
+  else
+    hipLaunchKernelGGL((act_fwd_kernel<bf16>), grid, block, 0, stream, T, I, gated, act, (const bf16*)pre, (bf16*)hid);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+int lt_act_backward(int64_t T, int64_t I, int gated, int act, int dtype, const void* pre, const void* dhid, void* dpre,
+                    hipStream_t stream) {
+  LT_REQUIRE(T > 0 && I > 0 && pre && dhid && dpre, LT_ERR_BAD_ARG, "activation backward: bad arguments");
+  dim3 grid(blocks_for(T * I, 256)), block(256);
+  if (dtype == LT_F32)
+    hipLaunchKernelGGL((act_bwd_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre,
+                       (const float*)dhid, (float*)dpre);
+  else
+    hipLaunchKernelGGL((act_bwd_kernel<bf16>), grid, block, 0, stream, T, I, gated, act, (const bf16*)pre,
+                       (const bf16*)dhid, (bf16*)dpre);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+int lt_dropout_cast(int64_t n, int in_dtype, const void* in, int out_dtype, void* out, const DropoutParams& drop,
+                    hipStream_t stream) {
+  LT_REQUIRE(n > 0 && in && out, LT_ERR_BAD_ARG, "dropout: bad arguments");
+  dim3 grid(blocks_for(n, 256)), block(256);
+  const int key = (in_dtype == LT_BF16) * 2 + (out_dtype == LT_BF16);
+  switch (key) {
+    case 0: hipLaunchKernelGGL((dropout_cast_kernel<float, float>), grid, block, 0, stream, n, (const float*)in, (float*)out, drop); break;
+    case 1: hipLaunchKernelGGL((dropout_cast_kernel<float, bf16>), grid, block, 0, stream, n, (const float*)in, (bf16*)out, drop); break;
+    case 2: hipLaunchKernelGGL((dropout_cast_kernel<bf16, float>), grid, block, 0, stream, n, (const bf16*)in, (float*)out, drop); break;
+    default: hipLaunchKernelGGL((dropout_cast_kernel<bf16, bf16>), grid, block, 0, stream, n, (const bf16*)in, (bf16*)out, drop); break;
+  }
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+int lt_dropout_mask_launch(int64_t n, uint8_t* keep, const DropoutParams& drop, hipStream_t stream) {
+  LT_REQUIRE(n > 0 && keep, LT_ERR_BAD_ARG, "dropout mask: bad arguments");
+  hipLaunchKernelGGL(dropout_mask_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, n, keep, drop);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}

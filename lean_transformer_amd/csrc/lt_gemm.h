@@ -1,0 +1,238 @@
+// GEMM problem description and fused epilogues shared by the any-shape kernel and the tiled bf16 MFMA kernel.
+#pragma once
+#include "lt_common.h"
+
+// C[m, n] = sum over up to two K segments of  sum_k A_s(m, k) * B_s(n, k)   (fp32 accumulation), then one epilogue.
+// The second segment carries the low-rank term of a generalized linear layer without a second pass over C.
+struct GemmOperand {
+  const void* ptr;
+  int64_t ld;   // leading dimension in elements
+  int kmajor;   // 1: element (i, k) at ptr[i * ld + k]; 0: at ptr[k * ld + i]
+};
+
+enum EpiKind {
+  EPI_STORE = 0,    // out[m, n] = acc + bias[n]
+  EPI_ACT_FWD = 1,  // up-projection: store pre-activation, apply (gated) activation, store hidden
+  EPI_ACT_BWD = 2,  // d(hidden) -> d(pre-activation) (both halves when gated) and the re-materialised hidden
+  EPI_OUT = 3       // down-projection: + bias, dropout, + residual, store y
+};
+
+struct EpiParams {
+  const float* bias;  // indexed by the global output column; may be null
+  // EPI_STORE
+  void* out;
+  int64_t ldo;
+  int out_dtype;
+  // EPI_ACT_FWD / EPI_ACT_BWD
+  void* pre;          // ACT_FWD: written, ACT_BWD: read.  [M, gated ? 2I : I]
+  int64_t ld_pre;
+  void* hid;          // [M, I], written (may be null in ACT_BWD)
+  int64_t ld_hid;
+  void* dpre;         // ACT_BWD: [M, gated ? 2I : I], written
+  int gated;
+  int act;
+  int64_t inter;      // I
+  // EPI_OUT
+  const void* x;      // residual input [M, ldy] (null = no residual)
+  void* y;            // [M, ldy]
+  int64_t ldy;        // row width of x / y; element (m, n) draws dropout word m * ldy + n
+  DropoutParams drop;
+};
+
+// Block-sparse operand walk (any-shape kernel only).  Workgroups with the same blockIdx.z form one group:
+//   SPARSE_FWD  group = output block ob:  Y[:, ob] = sum_k X[:, ib_k] W4[ib_k, a_k]^T,  forward_indices[ob, k] = ib_k * A + a_k
+//   SPARSE_DX   group = input block ib:   dX[:, ib] = sum_a dY[:, ob_a] W4[ib, a],       ob_a = backward_indices[ib, a]
+//   SPARSE_DW   group = weight block (ib, a): dW4[ib, a] = dY[:, ob_a]^T X[:, ib]
+// W4 = the native weight [in_features, A, block] read as [in_blocks, A, block (output row), block (input column)].
+// In FWD / DX an optional dense low-rank segment (A[1], B[1], K[1] of the enclosing problem) is appended.
+enum SparseMode { SPARSE_NONE = 0, SPARSE_FWD = 1, SPARSE_DX = 2, SPARSE_DW = 3 };
+
+struct SparseWalk {
+  int mode;
+  int block;           // b
+  int blocks_per_out;  // K
+  int blocks_per_in;   // A
+  const int32_t* forward_indices;
+  const int64_t* backward_indices;
+  const void* act;     // FWD: X [M, in]; DX / DW: dY [M(tokens), out]
+  int64_t ld_act;
+  const void* weight;  // FWD / DX: W4
+  const void* act2;    // DW: X [tokens, in]
+  int64_t ld_act2;
+  int64_t tokens;      // DW: reduction length
+};
+
+struct GemmProblem {
+  int64_t M;
+  int64_t N;  // output columns; for a gated EPI_ACT_FWD this counts gate columns (I) and B has 2I rows
+  int nseg;
+  int64_t K[2];
+  GemmOperand A[2], B[2];
+  EpiParams epi;
+  SparseWalk sp;  // sp.mode == SPARSE_NONE for a dense problem
+};
+
+// ---------------------------------------------------------------------------------------------------------------------
+// per-element epilogues.  TC: compute dtype (pre-activation, hidden, gradients of them), TX: dtype of x / y.
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename TO> __device__ __forceinline__ void epi_store(const EpiParams& e, int64_t m, int64_t n, float v) {
+  if (e.bias) v += e.bias[n];
+  stf(reinterpret_cast<TO*>(e.out), m * e.ldo + n, v);
+}
+
+template <typename TC> __device__ __forceinline__ void epi_act_fwd(const EpiParams& e, int64_t m, int64_t n, float v) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  if (e.bias) v += e.bias[n];
+  TC pv = from_f32<TC>(v);
+  reinterpret_cast<TC*>(e.pre)[m * e.ld_pre + n] = pv;
+  stf(reinterpret_cast<TC*>(e.hid), m * e.ld_hid + n, act_value<PRECISE>(e.act, to_f32(pv)));
+}
+
+// gated: column n of the gate half pairs with column I + n of the linear half
+template <typename TC>
+__device__ __forceinline__ void epi_act_fwd_gated(const EpiParams& e, int64_t m, int64_t n, float vg, float vl) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  if (e.bias) {
+    vg += e.bias[n];
+    vl += e.bias[e.inter + n];
+  }
+  TC pg = from_f32<TC>(vg), pl = from_f32<TC>(vl);
+  TC* pre = reinterpret_cast<TC*>(e.pre);
+  pre[m * e.ld_pre + n] = pg;
+  pre[m * e.ld_pre + e.inter + n] = pl;
+  stf(reinterpret_cast<TC*>(e.hid), m * e.ld_hid + n, act_value<PRECISE>(e.act, to_f32(pg)) * to_f32(pl));
+}
+
+template <typename TC> __device__ __forceinline__ void epi_act_bwd(const EpiParams& e, int64_t m, int64_t n, float dh) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  const TC* pre = reinterpret_cast<const TC*>(e.pre);
+  TC* dpre = reinterpret_cast<TC*>(e.dpre);
+  TC* hid = reinterpret_cast<TC*>(e.hid);
+  float a, da;
+  if (e.gated) {
+    float pg = to_f32(pre[m * e.ld_pre + n]), pl = to_f32(pre[m * e.ld_pre + e.inter + n]);
+    act_eval<PRECISE>(e.act, pg, a, da);
+    stf(dpre, m * e.ld_pre + n, dh * pl * da);
+    stf(dpre, m * e.ld_pre + e.inter + n, dh * a);
+    if (hid) stf(hid, m * e.ld_hid + n, a * pl);
+  } else {
+    float p = to_f32(pre[m * e.ld_pre + n]);
+    act_eval<PRECISE>(e.act, p, a, da);
+    stf(dpre, m * e.ld_pre + n, dh * da);
+    if (hid) stf(hid, m * e.ld_hid + n, a);
+  }
+}
+
+template <typename TX> __device__ __forceinline__ void epi_out(const EpiParams& e, int64_t m, int64_t n, float v) {
+  if (e.bias) v += e.bias[n];
+  int64_t idx = m * e.ldy + n;
+  if (e.drop.p > 0.f) v = dropout_keep(e.drop, idx) ? v * e.drop.scale : 0.f;
+  if (e.x) v += ldf(reinterpret_cast<const TX*>(e.x), idx);
+  stf(reinterpret_cast<TX*>(e.y), idx, v);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// the same epilogues on 8 consecutive columns n .. n + 7 of row m (n a multiple of 8, all leading dimensions multiples
+// of 8): 16-byte global accesses, one Philox block per 4 elements.  Used by the tiled bf16 kernel (TC = bf16).
+// ---------------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void add_bias8(const float* bias, int64_t n, float (&v)[8]) {
+  if (bias) {
+    float b[8];
+    load8(bias + n, b);
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] += b[i];
+  }
+}
+
+__device__ __forceinline__ void epi_store8(const EpiParams& e, int64_t m, int64_t n, float (&v)[8]) {
+  add_bias8(e.bias, n, v);
+  if (e.out_dtype == LT_F32) store8(reinterpret_cast<float*>(e.out) + m * e.ldo + n, v);
+  else store8(reinterpret_cast<bf16*>(e.out) + m * e.ldo + n, v);
+}
+
+__device__ __forceinline__ void epi_act_fwd8(const EpiParams& e, int64_t m, int64_t n, float (&v)[8]) {
+  add_bias8(e.bias, n, v);
+  float h[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    v[i] = to_f32((bf16)v[i]);  // the activation sees the stored (rounded) pre-activation, as backward will
+    h[i] = act_value<false>(e.act, v[i]);
+  }
+  store8(reinterpret_cast<bf16*>(e.pre) + m * e.ld_pre + n, v);
+  store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, h);
+}
+
+__device__ __forceinline__ void epi_act_fwd_gated8(const EpiParams& e, int64_t m, int64_t n, float (&vg)[8], float (&vl)[8]) {
+  add_bias8(e.bias, n, vg);
+  add_bias8(e.bias, e.inter + n, vl);
+  float h[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    vg[i] = to_f32((bf16)vg[i]);
+    vl[i] = to_f32((bf16)vl[i]);
+    h[i] = act_value<false>(e.act, vg[i]) * vl[i];
+  }
+  bf16* pre = reinterpret_cast<bf16*>(e.pre) + m * e.ld_pre + n;
+  store8(pre, vg);
+  store8(pre + e.inter, vl);
+  store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, h);
+}
+
+__device__ __forceinline__ void epi_act_bwd8(const EpiParams& e, int64_t m, int64_t n, const float (&dh)[8]) {
+  const bf16* pre = reinterpret_cast<const bf16*>(e.pre) + m * e.ld_pre + n;
+  bf16* dpre = reinterpret_cast<bf16*>(e.dpre) + m * e.ld_pre + n;
+  float pg[8], a[8], da[8], o[8];
+  load8(pre, pg);
+#pragma unroll
+  for (int i = 0; i < 8; i++) act_eval<false>(e.act, pg[i], a[i], da[i]);
+  if (e.gated) {
+    float pl[8];
+    load8(pre + e.inter, pl);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * pl[i] * da[i];
+    store8(dpre, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * a[i];
+    store8(dpre + e.inter, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] *= pl[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * da[i];
+    store8(dpre, o);
+  }
+  if (e.hid) store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, a);
+}
+
+template <typename TX> __device__ __forceinline__ void epi_out8(const EpiParams& e, int64_t m, int64_t n, float (&v)[8]) {
+  add_bias8(e.bias, n, v);
+  const int64_t idx = m * e.ldy + n;
+  if (e.drop.p > 0.f) {
+    bool k0[4], k1[4];
+    dropout_keep4(e.drop, idx, k0);
+    dropout_keep4(e.drop, idx + 4, k1);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[i] = k0[i] ? v[i] * e.drop.scale : 0.f;
+      v[i + 4] = k1[i] ? v[i + 4] * e.drop.scale : 0.f;
+    }
+  }
+  if (e.x) {
+    float r[8];
+    load8(reinterpret_cast<const TX*>(e.x) + idx, r);
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] += r[i];
+  }
+  store8(reinterpret_cast<TX*>(e.y) + idx, v);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// launchers (defined in gemm_generic.hip / gemm_mfma_bf16.hip)
+// ---------------------------------------------------------------------------------------------------------------------
+// any shape, fp32 or bf16 operands (dtype), fp32 MFMA arithmetic.  io_dtype: dtype of x / y for EPI_OUT.
+int lt_launch_gemm_generic(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);
+// true when the tiled bf16 kernel handles this problem (operand layouts, alignment, tile divisibility)
+bool lt_gemm_mfma_supported(const GemmProblem& p, int kind);
+int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_t stream);
+// picks the tiled kernel when it applies and dtype is bf16, else the any-shape kernel
+int lt_launch_gemm(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);

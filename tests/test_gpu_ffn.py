@@ -1,0 +1,346 @@
+"""GPU parity of the whole LeanFFN block (module -> autograd.Function -> C ABI -> HIP kernels) against the CPU oracle.
+
+Small and medium shapes are checked against the oracle on the CPU; the configurations at full benchmark size are checked
+against the same oracle code evaluated in fp32 on GPU tensors (the oracle is plain PyTorch and device-agnostic) and through
+size-independent properties.  Bars: fp32 max relative error <= 1e-4; bf16 <= 2e-2 with cosine >= 0.9999, on y, dx and every
+parameter gradient."""
+import pytest
+import torch
+import torch.nn as nn
+
+import lean_transformer_amd as lt
+from conftest import assert_close
+from helpers import dropout_mask, generator_position, module_tensors, oracle_params, run_oracle
+from lean_transformer_amd.utils import ACT2FN
+from oracle import ffn as offn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _run_module(ffn, x, dy):
+    """(y, dx, grads of module_tensors(ffn))"""
+    x = x.detach().clone().requires_grad_(True)
+    y = ffn(x)
+    grads = torch.autograd.grad(y, [x, *module_tensors(ffn)], dy)
+    return y.detach(), grads[0], list(grads[1:])
+
+
+def _compare(ffn, x_cpu, dy_cpu, dtype, oracle_device="cpu", mask=None):
+    p = oracle_params(ffn, oracle_device)
+    y_ref, dx_ref, g_ref = run_oracle(p, x_cpu.float().to(oracle_device), dy_cpu.float().to(oracle_device), mask)
+    y, dx, g = _run_module(ffn, x_cpu.to(DEV), dy_cpu.to(DEV))
+    assert_close(y, y_ref, dtype, "y")
+    assert_close(dx, dx_ref, dtype, "dx")
+    assert len(g) == len(g_ref)
+    for i, (a, b) in enumerate(zip(g, g_ref)):
+        assert_close(a, b, dtype, f"param grad {i}")
+
+
+def test_ffn_simple_stacked():
+    """reference tests/test_ffn.py:33-86: LeanFFN(32, 128) applied 4 times, outputs / input grads / parameter grads"""
+    torch.manual_seed(0)
+    ffn = lt.LeanFFN(32, 128).to(DEV)
+    p = oracle_params(ffn)
+    x = torch.rand(4, 128, 32)
+    xr = x.clone().requires_grad_(True)
+    out_ref = xr
+    for _ in range(4):
+        out_ref = offn.plain_ffn(out_ref, p)
+    obj_ref = (out_ref * (out_ref + 1)).square().mean()
+    ref = torch.autograd.grad(obj_ref, [xr, *p.tensors()])
+    xd = x.to(DEV).requires_grad_(True)
+    out = xd
+    for _ in range(4):
+        out = ffn(out)
+    obj = (out * (out + 1)).square().mean()
+    got = torch.autograd.grad(obj, [xd, *module_tensors(ffn)])
+    assert_close(out, out_ref.detach(), torch.float32, "out")
+    for i, (a, b) in enumerate(zip(got, ref)):
+        assert_close(a, b, torch.float32, f"grad {i}")
+
+
+@pytest.mark.parametrize("adapter_dim,lowrank_dim,block_size,residual", [
+    (0, 0, 0, True), (0, 0, 0, False), (0, 0, 16, False), (4, 0, 0, True), (0, 4, 0, True), (2, 6, 0, False),
+    (6, 2, 16, True), (0, 2, 16, True), (1, 0, 16, False)])
+@pytest.mark.parametrize("gated", [True, False])
+def test_ffn_generalized_projections(adapter_dim, lowrank_dim, block_size, residual, gated):
+    """the grid of reference tests/test_ffn.py:150-241 (dim 32, pixelfly(16), gated, post-LN, shared low-rank + adapter)"""
+    torch.manual_seed(adapter_dim * 100 + lowrank_dim * 10 + block_size)
+    dim = 32
+    layout = f"pixelfly({block_size})" if block_size else None
+    n1 = 8 * dim if gated else 4 * dim
+    ffn = lt.LeanFFN(
+        dim, 4 * dim, gated=gated, post_layer_norm=True, layer_norm_eps=1e-5,
+        i2h_proj=lt.GeneralizedLinear(lt.GeneralizedMatrix(dim, n1, layout, lowrank_dim), adapter_dim),
+        h2o_proj=lt.GeneralizedLinear(lt.GeneralizedMatrix(4 * dim, dim, layout, lowrank_dim), adapter_dim),
+        residual=residual)
+    with torch.no_grad():
+        ffn.post_layer_norm.bias.normal_()
+        ffn.post_layer_norm.weight.uniform_(0.5, 1.5)
+        ffn.i2h_proj.bias.normal_(std=0.1)
+        ffn.h2o_proj.bias.normal_(std=0.1)
+        for proj in (ffn.i2h_proj, ffn.h2o_proj):
+            if proj.adapter_second is not None:
+                proj.adapter_second.normal_(std=0.1)
+    ffn = ffn.to(DEV)
+    x, dy = torch.rand(4, 37, dim), torch.randn(4, 37, dim)
+    p = oracle_params(ffn)
+    y_ref, dx_ref, _ = run_oracle(p, x, dy)
+    xd = x.to(DEV).requires_grad_(True)
+    y = ffn(xd)
+    names, params = zip(*ffn.named_parameters())
+    grads = torch.autograd.grad(y, [xd, *params], dy.to(DEV))
+    assert_close(y, y_ref, torch.float32, "y")
+    assert_close(grads[0], dx_ref, torch.float32, "dx")
+    # parameter gradients against autograd of the module's own plain-autograd path evaluated by the oracle: rebuild the
+    # oracle with leaves per module parameter (combined low-rank factors split back into shared part and adapter)
+    ref = _oracle_named_grads(ffn, x, dy)
+    for name, grad in zip(names, grads[1:]):
+        assert_close(grad, ref[name], torch.float32, name)
+
+
+def _oracle_named_grads(ffn, x, dy):
+    """gradients per named module parameter, from the CPU oracle with the low-rank factors concatenated from leaves"""
+    leaves = {n: t.detach().cpu().float().clone().requires_grad_(True) for n, t in ffn.named_parameters()}
+
+    def proj(prefix, module):
+        w = leaves[f"{prefix}.matrix.weight"]
+        firsts = [leaves[k] for k in (f"{prefix}.matrix.lowrank_first", f"{prefix}.adapter_first") if k in leaves]
+        seconds = [leaves[k] for k in (f"{prefix}.matrix.lowrank_second", f"{prefix}.adapter_second") if k in leaves]
+        fwd, bwd = module.matrix.forward_indices, module.matrix.backward_indices
+        return offn.LinearParams(w, leaves.get(f"{prefix}.bias"), torch.cat(firsts, 0) if firsts else None,
+                                 torch.cat(seconds, 1) if seconds else None, None if fwd is None else fwd.cpu(),
+                                 None if bwd is None else bwd.cpu(), out_features=module.out_features)
+
+    p = offn.FFNParams(leaves["pre_layer_norm.weight"], leaves["pre_layer_norm.bias"], proj("i2h_proj", ffn.i2h_proj),
+                       proj("h2o_proj", ffn.h2o_proj), leaves.get("post_layer_norm.weight"),
+                       leaves.get("post_layer_norm.bias"),
+                       offn.FFNConfig(gated=ffn.gated, ln_eps=ffn.pre_layer_norm.eps, residual=ffn.residual))
+    y = offn.plain_ffn(x, p)
+    names = list(leaves)
+    grads = torch.autograd.grad(y, [leaves[n] for n in names], dy)
+    return dict(zip(names, grads))
+
+
+@pytest.mark.parametrize("act", ["gelu_fused", "gelu", "relu", "silu"])
+@pytest.mark.parametrize("gated", [False, True])
+def test_ffn_activations_fp32(act, gated):
+    torch.manual_seed(1)
+    ffn = lt.LeanFFN(48, 80, activation=ACT2FN[act], gated=gated, layer_norm_eps=1e-5).to(DEV)
+    _compare(ffn, torch.randn(3, 21, 48), torch.randn(3, 21, 48), torch.float32)
+
+
+def test_ffn_dropout_behaviour():
+    """reference tests/test_ffn.py:244-272: without dropout two runs agree, with dropout they differ (forward and grad)"""
+    torch.manual_seed(0)
+    for dropout in (0.0, 0.5):
+        ffn = lt.LeanFFN(32, 128, post_layer_norm=True, gated=True, dropout=dropout).to(DEV)
+        x = torch.rand(4, 128, 32, device=DEV, requires_grad=True)
+        runs = []
+        for _ in range(2):
+            out = x
+            for _ in range(4):
+                out = ffn(out)
+            (grad,) = torch.autograd.grad(out.norm(), x)
+            runs.append((out.detach(), grad))
+        same_out = torch.allclose(runs[0][0], runs[1][0], rtol=1e-3, atol=1e-5)
+        same_grad = torch.allclose(runs[0][1], runs[1][1], rtol=1e-3, atol=1e-5)
+        assert same_out == (dropout == 0) and same_grad == (dropout == 0)
+        ffn.eval()  # dropout is active only in training mode (ffn.py:128,202)
+        assert torch.equal(ffn(x), ffn(x))
+
+
+@pytest.mark.parametrize("post_ln", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ffn_dropout_mask_parity(post_ln, dtype):
+    """the mask is never stored: forward epilogue and backward replay evaluate the same Philox stream.  Hand the oracle the
+    mask of that stream and compare everything; seeding the generator reproduces the run."""
+    torch.manual_seed(3)
+    hidden, inter, tokens = 256, 512, 300
+    ffn = lt.LeanFFN(hidden, inter, dropout=0.1, post_layer_norm=post_ln, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.i2h_proj.weight.normal_(std=0.05)
+        ffn.h2o_proj.weight.normal_(std=0.05)
+    ffn = ffn.to(DEV)
+    if dtype == torch.bfloat16:
+        ffn = ffn.to(torch.bfloat16)
+    x, dy = torch.randn(tokens, hidden), torch.randn(tokens, hidden)
+    torch.cuda.manual_seed(77)
+    seed, offset = generator_position(DEV)
+    y, dx, g = _run_module(ffn, x.to(DEV), dy.to(DEV))
+    assert generator_position(DEV)[1] == offset + tokens * hidden  # the stream advanced by one word per element
+    mask = dropout_mask(tokens, hidden, 0.1, seed, offset, torch.device(DEV)).cpu()
+    assert abs(mask.float().mean().item() - 0.9) < 0.01
+    p = oracle_params(ffn)
+    y_ref, dx_ref, g_ref = run_oracle(p, x, dy, mask)
+    assert_close(y, y_ref, dtype, "y")
+    assert_close(dx, dx_ref, dtype, "dx")
+    for i, (a, b) in enumerate(zip(g, g_ref)):
+        assert_close(a, b, dtype, f"param grad {i}")
+    if not post_ln:  # dropped outputs are exactly the residual, and their upstream gradient never reaches the weights
+        assert torch.equal(y.cpu()[~mask], x[~mask])
+    torch.cuda.manual_seed(77)
+    y2, dx2, _ = _run_module(ffn, x.to(DEV), dy.to(DEV))
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+
+
+def _c1():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(8, 512, 768, generator=g)
+    ffn = lt.LeanFFN(768, 3072, gated=True, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.i2h_proj.weight.copy_(torch.randn(6144, 768, generator=g) * 0.02)
+        ffn.h2o_proj.weight.copy_(torch.randn(768, 3072, generator=g) * 0.02)
+        ffn.i2h_proj.bias.zero_()
+        ffn.h2o_proj.bias.zero_()
+    dy = torch.randn(8, 512, 768, generator=g)
+    return ffn, x, dy
+
+
+def test_config1_fp32_against_cpu_oracle():
+    """BASELINE config 1: fp32, hidden 768, intermediate 3072, GeGLU, eps 1e-5, x [8, 512, 768]; oracle on the host cores"""
+    ffn, x, dy = _c1()
+    _compare(ffn.to(DEV), x, dy, torch.float32)
+
+
+@pytest.mark.parametrize("gated", [True, False])
+@pytest.mark.parametrize("tokens", [1024, 1000, 1])
+@pytest.mark.parametrize("io_dtype", [torch.float32, torch.bfloat16])
+def test_ffn_bf16_tiled_kernels_against_cpu_oracle(gated, tokens, io_dtype):
+    """bf16 weights, shapes the tiled MFMA kernels take (hidden, intermediate multiples of 256), ragged token counts"""
+    torch.manual_seed(tokens + gated)
+    hidden, inter = 512, 1024
+    ffn = lt.LeanFFN(hidden, inter, gated=gated, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.pre_layer_norm.weight.uniform_(0.5, 1.5)
+        ffn.pre_layer_norm.bias.normal_(std=0.2)
+        ffn.i2h_proj.bias.normal_(std=0.1)
+        ffn.h2o_proj.bias.normal_(std=0.1)
+    ffn = ffn.to(DEV).to(torch.bfloat16)
+    x, dy = torch.randn(tokens, hidden).to(io_dtype), torch.randn(tokens, hidden).to(io_dtype)
+    _compare(ffn, x, dy, torch.bfloat16)
+
+
+def test_ffn_autocast_fp32_master_weights():
+    """fp32 parameters under torch.autocast(bfloat16): GEMM operands are cast per call, gradients come back in fp32"""
+    torch.manual_seed(5)
+    ffn = lt.LeanFFN(256, 512, gated=True, layer_norm_eps=1e-5).to(DEV)
+    x, dy = torch.randn(260, 256), torch.randn(260, 256)
+    p = oracle_params(ffn)
+    y_ref, dx_ref, g_ref = run_oracle(p, x, dy)
+    xd = x.to(DEV).requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = ffn(xd)
+    grads = torch.autograd.grad(y, [xd, *module_tensors(ffn)], dy.to(DEV))
+    assert y.dtype == torch.float32 and all(g.dtype == torch.float32 for g in grads)
+    assert_close(y, y_ref, torch.bfloat16, "y")
+    assert_close(grads[0], dx_ref, torch.bfloat16, "dx")
+    for i, (a, b) in enumerate(zip(grads[1:], g_ref)):
+        assert_close(a, b, torch.bfloat16, f"param grad {i}")
+
+
+def test_custom_grad_switch_and_partial_grads():
+    """ffn_custom_grad is a live attribute (transformer.py:142-143 flips it): both paths agree; gradients that are not
+    required are not produced; the block runs under activation checkpointing"""
+    torch.manual_seed(9)
+    ffn = lt.LeanFFN(64, 128, gated=True, post_layer_norm=True, layer_norm_eps=1e-5).to(DEV)
+    x = torch.randn(5, 7, 64, device=DEV, requires_grad=True)
+    dy = torch.randn(5, 7, 64, device=DEV)
+    ffn.ffn_custom_grad = True
+    y1 = ffn(x)
+    g1 = torch.autograd.grad(y1, [x, *ffn.parameters()], dy)
+    ffn.ffn_custom_grad = False
+    y2 = ffn(x)
+    g2 = torch.autograd.grad(y2, [x, *ffn.parameters()], dy)
+    assert_close(y1, y2, torch.float32, "y")
+    for a, b in zip(g1, g2):
+        assert_close(a, b, torch.float32, "grad")
+    ffn.ffn_custom_grad = True
+    for prm in ffn.parameters():
+        prm.requires_grad_(False)
+    ffn.h2o_proj.weight.requires_grad_(True)
+    ffn(x.detach()).backward(dy)
+    assert ffn.h2o_proj.weight.grad is not None and ffn.i2h_proj.weight.grad is None
+    assert_close(ffn.h2o_proj.weight.grad, g1[1 + list(dict(ffn.named_parameters())).index("h2o_proj.weight")],
+                 torch.float32, "h2o grad alone")
+    for prm in ffn.parameters():
+        prm.requires_grad_(True)
+    from torch.utils.checkpoint import checkpoint
+    y3 = checkpoint(ffn, x, use_reentrant=False)
+    g3 = torch.autograd.grad(y3, [x, ffn.i2h_proj.weight], dy)
+    assert_close(g3[0], g1[0], torch.float32, "dx under checkpoint")
+
+
+def _headline(hidden, inter, gated, std, dropout, shape, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(*shape, hidden, generator=g)
+    n1 = 2 * inter if gated else inter
+    ffn = lt.LeanFFN(hidden, inter, gated=gated, layer_norm_eps=1e-5, dropout=dropout)
+    with torch.no_grad():
+        ffn.i2h_proj.weight.copy_(torch.randn(n1, hidden, generator=g) * std)
+        ffn.h2o_proj.weight.copy_(torch.randn(hidden, inter, generator=g) * std)
+        ffn.i2h_proj.bias.zero_()
+        ffn.h2o_proj.bias.zero_()
+    dy = torch.randn(*shape, hidden, generator=g)
+    return ffn.to(DEV).to(torch.bfloat16), x, dy
+
+
+def _full_size_checks(ffn, x, dy, mask_p):
+    tokens, hidden = x.shape[0] * x.shape[1], x.shape[-1]
+    torch.cuda.manual_seed(0)
+    seed, offset = generator_position(DEV)
+    y, dx, g = _run_module(ffn, x.to(DEV), dy.to(DEV))
+    mask = dropout_mask(tokens, hidden, mask_p, seed, offset, torch.device(DEV)) if mask_p > 0 else None
+    # (1) the oracle, evaluated in fp32 on the GPU, on the bf16-rounded weights
+    p = oracle_params(ffn, DEV)
+    y_ref, dx_ref, g_ref = run_oracle(p, x.to(DEV), dy.to(DEV), mask)
+    assert_close(y, y_ref, torch.bfloat16, "y")
+    assert_close(dx, dx_ref, torch.bfloat16, "dx")
+    for i, (a, b) in enumerate(zip(g, g_ref)):
+        assert_close(a, b, torch.bfloat16, f"param grad {i}")
+    del p, y_ref, dx_ref, g_ref
+    # (2) rows are independent: 128 rows through the oracle on the CPU
+    rows = torch.randperm(tokens, generator=torch.Generator().manual_seed(1))[:128]
+    p_cpu = oracle_params(ffn, "cpu")
+    x2, dy2 = x.reshape(tokens, hidden)[rows], dy.reshape(tokens, hidden)[rows]
+    y_cpu, dx_cpu, _ = run_oracle(p_cpu, x2, dy2, None if mask is None else mask.cpu()[rows])
+    assert_close(y.reshape(tokens, hidden)[rows.to(DEV)], y_cpu, torch.bfloat16, "y rows")
+    assert_close(dx.reshape(tokens, hidden)[rows.to(DEV)], dx_cpu, torch.bfloat16, "dx rows")
+    # (3) weight gradients are sums over tokens: two halves of the batch add up to the whole (no dropout in this check,
+    #     each half draws its own stream)
+    if mask is None:
+        half = tokens // 2
+        xf, dyf = x.reshape(tokens, hidden), dy.reshape(tokens, hidden)
+        _, _, ga = _run_module(ffn, xf[:half].to(DEV), dyf[:half].to(DEV))
+        _, _, gb = _run_module(ffn, xf[half:].to(DEV), dyf[half:].to(DEV))
+        for i, (whole, a, b) in enumerate(zip(g, ga, gb)):
+            assert_close(whole.float(), a.float() + b.float(), torch.bfloat16, f"additivity of param grad {i}")
+
+
+def test_config2_bf16_full_size():
+    """BASELINE config 2: bf16, hidden 2048, intermediate 8192, plain GELU, dropout 0.1, x [4, 2048, 2048]"""
+    ffn, x, dy = _headline(2048, 8192, False, 0.02, 0.1, (4, 2048))
+    _full_size_checks(ffn, x, dy, 0.1)
+
+
+def test_config3_bf16_full_size_headline():
+    """BASELINE config 3 (headline): bf16, hidden 4096, intermediate 16384, GeGLU, x [2, 2048, 4096], weights ~N(0, 0.01)"""
+    ffn, x, dy = _headline(4096, 16384, True, 0.01, 0.0, (2, 2048))
+    _full_size_checks(ffn, x, dy, 0.0)
+
+
+def test_saved_activation_memory_matches_reference_keep_set():
+    """what stays alive between forward and backward is x (caller-owned), the pre-activation and 8 bytes of LayerNorm
+    statistics per token -- the reference's keep-set (ffn.py:210-216)"""
+    ffn, x, dy = _headline(1024, 4096, True, 0.02, 0.0, (2, 512))
+    xd = x.to(DEV).requires_grad_(True)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    y = ffn(xd)
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before
+    tokens = 1024
+    expected = tokens * 1024 * 4 + tokens * 2 * 4096 * 2 + tokens * 8  # y (fp32) + pre-activation (bf16) + stats
+    assert held <= expected + (1 << 20), (held, expected)
+    y.backward(dy.to(DEV))

@@ -1,0 +1,248 @@
+"""GPU parity of the individual kernels, called through the C ABI (ctypes): GEMM cores in every operand layout, LayerNorm
+forward / backward, activations, dropout mask, block-sparse matmul (against the reference's golden vectors) and the
+generalized linear layer.  Bars: fp32 max relative error <= 1e-4; bf16 <= 2e-2 with cosine >= 0.9999."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import lean_transformer_amd as lt
+from conftest import assert_close, rel_err
+from helpers import dropout_mask
+from lean_transformer_amd import _native as nat
+from oracle import blocksparse as obs
+from oracle import ffn as offn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+GOLDEN = np.load(os.path.join(os.path.dirname(__file__), "golden", "blocksparse_golden.npz"))
+
+
+def _gemm(a, b, a_kmajor, b_kmajor, m, n, k, c_dtype, force_generic):
+    c = torch.empty(m, n, dtype=c_dtype, device=DEV)
+    nat.check(nat.lib().lt_gemm(nat.dtype_code(a.dtype), m, n, k, nat.ptr(a), int(a_kmajor), nat.ptr(b), int(b_kmajor),
+                                nat.dtype_code(c_dtype), nat.ptr(c), int(force_generic), nat.current_stream(c.device)),
+              "lt_gemm")
+    return c
+
+
+def _operands(m, n, k, a_kmajor, b_kmajor, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).to(dtype)
+    b = torch.randn(n, k, generator=g).to(dtype)
+    ref = a.double() @ b.double().t()
+    a_dev = (a if a_kmajor else a.t().contiguous()).to(DEV)
+    b_dev = (b if b_kmajor else b.t().contiguous()).to(DEV)
+    return a_dev, b_dev, ref
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("a_kmajor,b_kmajor", [(True, True), (True, False), (False, False), (False, True)])
+@pytest.mark.parametrize("m,n,k", [(70, 45, 33), (300, 260, 130), (1, 1, 1), (128, 128, 16)])
+def test_gemm_any_shape_kernel(dtype, a_kmajor, b_kmajor, m, n, k):
+    a, b, ref = _operands(m, n, k, a_kmajor, b_kmajor, dtype, seed=m + n + k)
+    c = _gemm(a, b, a_kmajor, b_kmajor, m, n, k, torch.float32, force_generic=True)
+    assert rel_err(c, ref) <= 1e-5  # fp32 MFMA on exactly representable inputs
+
+
+@pytest.mark.parametrize("a_kmajor,b_kmajor", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("m,n,k", [(512, 512, 256), (256, 768, 64), (1024, 256, 1024)])
+@pytest.mark.parametrize("c_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_tiled_bf16_kernel(a_kmajor, b_kmajor, m, n, k, c_dtype):
+    a, b, ref = _operands(m, n, k, a_kmajor, b_kmajor, torch.bfloat16, seed=m + 2 * n + 3 * k)
+    c = _gemm(a, b, a_kmajor, b_kmajor, m, n, k, c_dtype, force_generic=False)
+    if c_dtype == torch.float32:
+        assert rel_err(c, ref) <= 1e-5
+    else:
+        assert_close(c, ref.float(), torch.bfloat16, "c")
+    # and it agrees with the any-shape kernel to fp32 summation-order noise
+    c2 = _gemm(a, b, a_kmajor, b_kmajor, m, n, k, torch.float32, force_generic=True)
+    assert rel_err(c.float(), c2) <= (1e-5 if c_dtype == torch.float32 else 1e-2)
+
+
+def test_gemm_tiled_bf16_ragged_rows_and_reduction():
+    # k-major A with a ragged row count (rows past M are clamped on load, never stored)
+    a, b, ref = _operands(300, 256, 128, True, True, torch.bfloat16, seed=1)
+    assert rel_err(_gemm(a, b, True, True, 300, 256, 128, torch.float32, False), ref) <= 1e-5
+    a, b, ref = _operands(777, 512, 192, True, False, torch.bfloat16, seed=2)
+    assert rel_err(_gemm(a, b, True, False, 777, 512, 192, torch.float32, False), ref) <= 1e-5
+    # both operands mn-major with a reduction length that is not a multiple of the 64-wide k-step (zero-filled tail)
+    a, b, ref = _operands(256, 512, 200, False, False, torch.bfloat16, seed=3)
+    assert rel_err(_gemm(a, b, False, False, 256, 512, 200, torch.float32, False), ref) <= 1e-5
+    a, b, ref = _operands(512, 256, 1000, False, False, torch.bfloat16, seed=4)
+    assert rel_err(_gemm(a, b, False, False, 512, 256, 1000, torch.float32, False), ref) <= 1e-5
+
+
+@pytest.mark.parametrize("tokens,hidden", [(37, 32), (64, 768), (9, 4096), (3, 10), (5, 8192), (2, 8200)])
+@pytest.mark.parametrize("x_dtype,y_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.bfloat16)])
+def test_layernorm_forward(tokens, hidden, x_dtype, y_dtype):
+    g = torch.Generator().manual_seed(tokens * hidden)
+    x = (torch.randn(tokens, hidden, generator=g) * 2 + 0.5).to(x_dtype)
+    w, b = torch.rand(hidden, generator=g) + 0.5, torch.randn(hidden, generator=g)
+    ref = F.layer_norm(x.float(), (hidden,), w, b, 1e-5)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    y = torch.empty(tokens, hidden, dtype=y_dtype, device=DEV)
+    stats = torch.empty(tokens, 2, device=DEV)
+    nat.check(nat.lib().lt_layernorm_forward(tokens, hidden, 1e-5, nat.dtype_code(x_dtype), nat.ptr(xd), nat.ptr(wd),
+                                             nat.ptr(bd), nat.dtype_code(y_dtype), nat.ptr(y), nat.ptr(stats),
+                                             nat.current_stream(y.device)), "lt_layernorm_forward")
+    assert_close(y, ref, y_dtype, "y")
+    assert torch.allclose(stats[:, 0].cpu(), x.float().mean(-1), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(stats[:, 1].cpu(), torch.rsqrt(x.float().var(-1, unbiased=False) + 1e-5), rtol=1e-4)
+
+
+@pytest.mark.parametrize("tokens,hidden", [(37, 32), (300, 768), (2100, 256), (3, 10), (4, 8192)])
+@pytest.mark.parametrize("x_dtype,dy_dtype,dx_dtype", [(torch.float32, torch.float32, torch.float32),
+                                                       (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                                       (torch.float32, torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_layernorm_backward(tokens, hidden, x_dtype, dy_dtype, dx_dtype, with_residual):
+    g = torch.Generator().manual_seed(tokens + hidden)
+    x = (torch.randn(tokens, hidden, generator=g) * 2 + 0.5).to(x_dtype)
+    dy = torch.randn(tokens, hidden, generator=g).to(dy_dtype)
+    res = torch.randn(tokens, hidden, generator=g).to(dx_dtype)
+    w = torch.rand(hidden, generator=g) + 0.5
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    br = torch.zeros(hidden, dtype=torch.float64, requires_grad=True)
+    F.layer_norm(xr, (hidden,), wr, br, 1e-5).backward(dy.double())
+    ref_dx = xr.grad + (res.double() if with_residual else 0)
+    xd, dyd, wd, resd = x.to(DEV), dy.to(DEV), w.to(DEV), res.to(DEV)
+    stats = torch.stack([x.float().mean(-1), torch.rsqrt(x.float().var(-1, unbiased=False) + 1e-5)], 1).to(DEV)
+    dx = torch.empty(tokens, hidden, dtype=dx_dtype, device=DEV)
+    dw, db = torch.empty(hidden, device=DEV), torch.empty(hidden, device=DEV)
+    lib = nat.lib()
+    ws = nat.workspace(lib.lt_layernorm_backward_workspace_bytes(tokens, hidden), torch.device(DEV))
+    nat.check(lib.lt_layernorm_backward(tokens, hidden, nat.dtype_code(x_dtype), nat.ptr(xd), nat.ptr(stats), nat.ptr(wd),
+                                        nat.dtype_code(dy_dtype), nat.ptr(dyd), nat.dtype_code(dx_dtype),
+                                        nat.ptr(resd) if with_residual else None, nat.ptr(dx), nat.ptr(dw), nat.ptr(db),
+                                        nat.ptr(ws), ws.numel(), nat.current_stream(dx.device)), "lt_layernorm_backward")
+    assert_close(dx, ref_dx.float(), dx_dtype, "dx")
+    assert_close(dw, wr.grad.float(), torch.float32, "dweight")
+    assert_close(db, br.grad.float(), torch.float32, "dbias")
+
+
+@pytest.mark.parametrize("act", ["gelu_fused", "gelu", "relu", "silu"])
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_activation_forward_backward(act, gated, dtype):
+    from lean_transformer_amd.utils import ACT_KINDS
+    tokens, inter = 33, 70
+    g = torch.Generator().manual_seed(5)
+    pre = (torch.randn(tokens, 2 * inter if gated else inter, generator=g) * 3).to(dtype)
+    dh = torch.randn(tokens, inter, generator=g).to(dtype)
+    pr = pre.double().requires_grad_(True)
+    href = offn.apply_activation(pr, act, gated)
+    (dpre_ref,) = torch.autograd.grad(href, pr, dh.double())
+    pd, dhd = pre.to(DEV), dh.to(DEV)
+    hid, dpre = torch.empty_like(dhd), torch.empty_like(pd)
+    lib = nat.lib()
+    nat.check(lib.lt_activation_forward(tokens, inter, int(gated), ACT_KINDS[act], nat.dtype_code(dtype), nat.ptr(pd),
+                                        nat.ptr(hid), nat.current_stream(pd.device)), "lt_activation_forward")
+    nat.check(lib.lt_activation_backward(tokens, inter, int(gated), ACT_KINDS[act], nat.dtype_code(dtype), nat.ptr(pd),
+                                         nat.ptr(dhd), nat.ptr(dpre), nat.current_stream(pd.device)), "lt_activation_backward")
+    assert_close(hid, href.detach().float(), dtype, "hid")
+    assert_close(dpre, dpre_ref.float(), dtype, "dpre")
+
+
+def test_dropout_mask_properties():
+    dev = torch.device(DEV)
+    m1 = dropout_mask(512, 768, 0.1, seed=1234, offset=0, device=dev)
+    assert abs(m1.float().mean().item() - 0.9) < 5e-3
+    assert torch.equal(m1, dropout_mask(512, 768, 0.1, 1234, 0, dev))          # a pure function of (seed, offset, index)
+    assert not torch.equal(m1, dropout_mask(512, 768, 0.1, 1234, 4, dev))      # another stream offset
+    assert not torch.equal(m1, dropout_mask(512, 768, 0.1, 1235, 0, dev))      # another seed
+    assert dropout_mask(16, 32, 0.0, 1, 0, dev).all()
+    # a higher drop probability drops a superset (same random words against a higher threshold)
+    m5 = dropout_mask(512, 768, 0.5, 1234, 0, dev)
+    assert abs(m5.float().mean().item() - 0.5) < 5e-3 and not (m5 & ~m1).any()
+
+
+@pytest.mark.parametrize("name", [str(n) for n in GOLDEN["names"]])
+def test_blocksparse_matmul_against_reference_golden(name):
+    x, w, dy = (torch.from_numpy(GOLDEN[f"{name}/{k}"]).to(DEV) for k in ("x", "w", "dy"))
+    fwd = torch.from_numpy(GOLDEN[f"{name}/forward_indices"]).to(DEV)
+    bwd = torch.from_numpy(GOLDEN[f"{name}/backward_indices"]).to(DEV)
+    y = lt.blocksparse_matmul(x, w, fwd)
+    dx, dw = lt.blocksparse_matmul_backward(dy, x, w, bwd)
+    assert_close(y, torch.from_numpy(GOLDEN[f"{name}/y"]), torch.float32, "y")
+    assert_close(dx, torch.from_numpy(GOLDEN[f"{name}/dx"]), torch.float32, "dx")
+    assert_close(dw, torch.from_numpy(GOLDEN[f"{name}/dw"]), torch.float32, "dw")
+    dx_only, empty = lt.blocksparse_matmul_backward(dy, x, w, bwd, weight_requires_grad=False)
+    assert empty.numel() == 0 and torch.equal(dx_only, dx)
+
+
+@pytest.mark.parametrize("out_f,in_f,block,stretch,dtype", [
+    (1024, 256, 64, True, torch.bfloat16), (256, 1024, 64, False, torch.bfloat16), (384, 96, 96 // 4, False, torch.float32),
+    (8192 // 4, 4096 // 4, 256, True, torch.float32)])
+def test_blocksparse_matmul_against_oracle(out_f, in_f, block, stretch, dtype):
+    """larger blocks than the golden vectors hold (64: the headline block size; 256: reference tests/test_butterfly.py)"""
+    layout = obs.pixelfly_layout(out_f, in_f, block_size=block, stretch=stretch)
+    fwd, bwd = obs.indices_from_layout(layout)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(3, 50, in_f, generator=g).to(dtype)
+    w = (torch.randn(in_f, bwd.shape[1], block, generator=g) * 0.1).to(dtype)
+    dy = torch.randn(3, 50, out_f, generator=g).to(dtype)
+    y_ref = obs.blocksparse_matmul(x.float(), w.float(), fwd)
+    dx_ref, dw_ref = obs.blocksparse_matmul_backward(dy.float(), x.float(), w.float(), bwd)
+    y = lt.blocksparse_matmul(x.to(DEV), w.to(DEV), torch.from_numpy(fwd).to(DEV))
+    dx, dw = lt.blocksparse_matmul_backward(dy.to(DEV), x.to(DEV), w.to(DEV), torch.from_numpy(bwd).to(DEV))
+    assert_close(y, y_ref, dtype, "y")
+    assert_close(dx, dx_ref, dtype, "dx")
+    assert_close(dw, dw_ref, dtype, "dw")
+
+
+@pytest.mark.parametrize("block_size,lowrank_dim,adapter_dim", [(0, 0, 0), (0, 60, 0), (0, 0, 4), (0, 60, 4), (8, 0, 0),
+                                                                (8, 60, 4)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_generalized_linear_against_oracle(block_size, lowrank_dim, adapter_dim, bias):
+    """the cases of reference tests/test_linear.py:79-137 (dim 128, pixelfly block 8, low-rank 60, adapter 4)"""
+    torch.manual_seed(1337)
+    dim = 128
+    layout = f"pixelfly(block_size={block_size})" if block_size else None
+    layer = lt.GeneralizedLinear(lt.GeneralizedMatrix(dim, dim, layout, lowrank_dim), adapter_dim, bias=bias)
+    with torch.no_grad():
+        if adapter_dim:
+            layer.adapter_second.normal_(std=0.1)
+        if bias:
+            layer.bias.normal_()
+    x = torch.rand(4, 5, dim)
+    dy = torch.randn(4, 5, dim)
+    from helpers import oracle_linear
+    p = oracle_linear(layer, "cpu", torch.float32)
+    xr = x.clone().requires_grad_(True)
+    y_ref = offn.linear_forward(xr.reshape(-1, dim), p).reshape(4, 5, dim)
+    ref_grads = torch.autograd.grad(y_ref, [xr, *p.tensors()], dy)
+    layer = layer.to(DEV)
+    xd = x.to(DEV).requires_grad_(True)
+    y = layer(xd)
+    names = [n for n, _ in layer.named_parameters()]
+    grads = torch.autograd.grad(y, [xd, *layer.parameters()], dy.to(DEV))
+    assert_close(y, y_ref.detach(), torch.float32, "y")
+    assert_close(grads[0], ref_grads[0], torch.float32, "dx")
+    got = dict(zip(names, grads[1:]))
+    ref = dict(zip(["weight"] + (["bias"] if bias else []) + (["first", "second"] if (lowrank_dim or adapter_dim) else []),
+                   ref_grads[1:]))
+    assert_close(got["matrix.weight"], ref["weight"], torch.float32, "dweight")
+    if bias:
+        assert_close(got["bias"], ref["bias"], torch.float32, "dbias")
+    if lowrank_dim and adapter_dim:  # combined factors: shared low-rank rows first, adapter rows after (linear.py:131-136)
+        assert_close(got["matrix.lowrank_first"], ref["first"][:lowrank_dim], torch.float32, "dlowrank_first")
+        assert_close(got["adapter_first"], ref["first"][lowrank_dim:], torch.float32, "dadapter_first")
+        assert_close(got["matrix.lowrank_second"], ref["second"][:, :lowrank_dim], torch.float32, "dlowrank_second")
+        assert_close(got["adapter_second"], ref["second"][:, lowrank_dim:], torch.float32, "dadapter_second")
+    elif lowrank_dim:
+        assert_close(got["matrix.lowrank_first"], ref["first"], torch.float32, "dlowrank_first")
+        assert_close(got["matrix.lowrank_second"], ref["second"], torch.float32, "dlowrank_second")
+    elif adapter_dim:
+        assert_close(got["adapter_first"], ref["first"], torch.float32, "dadapter_first")
+        assert_close(got["adapter_second"], ref["second"], torch.float32, "dadapter_second")
+
+
+def test_empty_batch():
+    layer = lt.GeneralizedLinear(lt.GeneralizedMatrix(32, 64)).to(DEV)
+    assert layer(torch.empty(0, 32, device=DEV)).shape == (0, 64)
+    ffn = lt.LeanFFN(32, 64).to(DEV)
+    assert ffn(torch.empty(2, 0, 32, device=DEV)).shape == (2, 0, 32)

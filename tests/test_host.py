@@ -1,0 +1,157 @@
+"""Host-side logic of the product package, on CPU: layouts / index tables against the reference's golden vectors, the module
+API and state_dict contract, activation mapping, and that the C-ABI library loads and exports what include/leanffn.h declares.
+No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import lean_transformer_amd as lt
+from lean_transformer_amd import _native as nat
+from lean_transformer_amd.blocksparse import layout as lay
+from lean_transformer_amd.utils import ACT2FN, activation_kind
+from oracle import ffn as offn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = np.load(os.path.join(os.path.dirname(__file__), "golden", "blocksparse_golden.npz"))
+
+
+@pytest.mark.parametrize("name", [str(n) for n in GOLDEN["names"]])
+def test_layout_and_indices_match_reference_golden(name):
+    out_f, in_f, block = (int(v) for v in GOLDEN[f"{name}/shape"])
+    layout = lay.get_blocksparse_layout(out_f, in_f, str(GOLDEN[f"{name}/desc"]))
+    assert layout.dtype == torch.bool and np.array_equal(layout.numpy(), GOLDEN[f"{name}/layout"])
+    fwd, bwd = lay.get_indices_from_layout(layout)
+    assert fwd.dtype == torch.int32 and bwd.dtype == torch.int64
+    assert np.array_equal(fwd.numpy(), GOLDEN[f"{name}/forward_indices"])
+    assert np.array_equal(bwd.numpy(), GOLDEN[f"{name}/backward_indices"])
+
+
+def test_layout_headline_shape_without_element_mask():
+    """32768 x 4096 with 64 x 64 blocks: 7 active blocks per row of the 64-cell butterfly, stretched or tiled"""
+    for stretch in (True, False):
+        up = lay.get_blocksparse_layout(32768, 4096, f"pixelfly(block_size=64, stretch={stretch})")
+        down = lay.get_blocksparse_layout(4096, 16384, f"pixelfly(block_size=64, stretch={stretch})")
+        assert up.shape == (512, 64) and down.shape == (64, 256)
+        assert up.sum(1).unique().tolist() == [7] and up.sum(0).unique().tolist() == [56]
+        assert down.sum(1).unique().tolist() == [28] and down.sum(0).unique().tolist() == [7]
+        fwd, bwd = lay.get_indices_from_layout(up)
+        assert fwd.shape == (512, 7) and bwd.shape == (64, 56) and fwd.max() == 7 * 512 - 1
+
+
+def test_layout_registry_and_errors():
+    @lay.register_blocksparse_layout("test_diag")
+    def make(out_features, in_features, foo):
+        smaller = min(out_features, in_features)
+        eye = torch.eye(smaller // foo, dtype=torch.bool)
+        return eye.repeat(out_features // smaller, in_features // smaller)
+
+    assert lay.get_blocksparse_layout(64, 32, "test_diag(foo=4)").float().mean().item() == pytest.approx(0.125)
+    with pytest.raises(ValueError):
+        lay.get_blocksparse_layout(64, 64, "nonexistent(1)")
+    with pytest.raises(AssertionError):
+        lay.get_indices_from_layout(torch.tensor([[True, False], [True, True]]))  # unbalanced
+    lay.REGISTERED_LAYOUTS.pop("test_diag")
+
+
+def test_constructor_defaults_and_state_dict_keys():
+    ffn = lt.LeanFFN(32, 128)
+    assert isinstance(ffn.i2h_proj, nn.Linear) and ffn.i2h_proj.out_features == 128
+    assert (ffn.gated, ffn.dropout, ffn.residual, ffn.ffn_custom_grad, ffn.post_layer_norm) == (False, 0.0, True, True, None)
+    assert ffn.pre_layer_norm.eps == 1e-12 and ffn.activation is ACT2FN["gelu_fused"]
+    assert sorted(ffn.state_dict()) == ["h2o_proj.bias", "h2o_proj.weight", "i2h_proj.bias", "i2h_proj.weight",
+                                        "pre_layer_norm.bias", "pre_layer_norm.weight"]
+    gated = lt.LeanFFN(32, 128, gated=True, post_layer_norm=True)
+    assert gated.i2h_proj.out_features == 256 and "post_layer_norm.weight" in gated.state_dict()
+    with pytest.raises(AssertionError):
+        lt.LeanFFN(32, 128, i2h_proj=nn.Linear(32, 64))
+    with pytest.raises(AssertionError):
+        lt.LeanFFN(32, 128, i2h_proj=nn.Sequential(nn.Linear(32, 128)))
+
+
+def test_generalized_linear_parameter_layout():
+    matrix = lt.GeneralizedMatrix(32, 256, "pixelfly(16)", lowrank_dim=4)
+    lin = lt.GeneralizedLinear(matrix, adapter_dim=2)
+    assert lin.weight is matrix.weight and tuple(matrix.weight.shape) == (32, 16, 16)
+    assert tuple(matrix.lowrank_first.shape) == (4, 32) and tuple(matrix.lowrank_second.shape) == (256, 4)
+    first, second = lin.get_combined_lowrank_components()
+    assert tuple(first.shape) == (6, 32) and tuple(second.shape) == (256, 6)
+    assert sorted(lin.state_dict()) == ["adapter_first", "adapter_second", "bias", "matrix.backward_indices",
+                                        "matrix.forward_indices", "matrix.layout", "matrix.lowrank_first",
+                                        "matrix.lowrank_second", "matrix.weight"]
+    dense = lt.GeneralizedLinear(lt.GeneralizedMatrix(32, 64))
+    assert tuple(dense.weight.shape) == (64, 32) and dense.matrix.forward_indices is None
+    assert dense.get_combined_lowrank_components() == (None, None)
+    with pytest.raises(NotImplementedError):
+        lt.GeneralizedMatrix(32, 64, "pixelfly(16)", blocksparse_backend="triton")
+    # a matrix shared between two layers is one parameter
+    shared = lt.GeneralizedMatrix(32, 32)
+    a, b = lt.GeneralizedLinear(shared, 2), lt.GeneralizedLinear(shared, 2)
+    assert a.weight is b.weight and a.adapter_first is not b.adapter_first
+
+
+def test_activation_mapping():
+    assert activation_kind(ACT2FN["gelu_fused"]) == "gelu_fused"
+    assert activation_kind(ACT2FN["gelu_new"]) == "gelu_fused"
+    assert activation_kind(ACT2FN["relu"]) == "relu" and activation_kind(ACT2FN["swish"]) == "silu"
+    assert activation_kind(torch.nn.functional.gelu) == "gelu" and activation_kind(nn.GELU(approximate="tanh")) == "gelu_fused"
+    with pytest.raises(NotImplementedError):
+        activation_kind(torch.sigmoid)
+    x = torch.linspace(-5, 5, 1000)
+    assert (ACT2FN["gelu_fused"](x) - torch.nn.functional.gelu(x)).abs().max().item() <= 5e-4  # reference tests/test_utils.py:25-29
+    assert torch.allclose(ACT2FN["gelu_fused"](x), offn.gelu_fused(x))
+
+
+def test_plain_autograd_path_on_cpu_matches_oracle():
+    """ffn_custom_grad=False is the reference's stock-op composition (ffn.py:69-85); with nn.Linear projections it runs
+    anywhere and must equal the oracle's plain_ffn"""
+    torch.manual_seed(0)
+    ffn = lt.LeanFFN(16, 32, gated=True, post_layer_norm=True, layer_norm_eps=1e-5, ffn_custom_grad=False)
+    x = torch.randn(2, 3, 16)
+    p = offn.FFNParams(ffn.pre_layer_norm.weight, ffn.pre_layer_norm.bias,
+                       offn.LinearParams(ffn.i2h_proj.weight, ffn.i2h_proj.bias, out_features=64),
+                       offn.LinearParams(ffn.h2o_proj.weight, ffn.h2o_proj.bias, out_features=16),
+                       ffn.post_layer_norm.weight, ffn.post_layer_norm.bias,
+                       offn.FFNConfig(gated=True, ln_eps=1e-5))
+    assert torch.allclose(ffn(x), offn.plain_ffn(x, p), rtol=1e-5, atol=1e-6)
+
+
+def test_custom_path_refuses_cpu_tensors():
+    ffn = lt.LeanFFN(16, 32)
+    with pytest.raises(RuntimeError, match="AMD GPUs only"):
+        ffn(torch.randn(2, 16))
+    with pytest.raises(RuntimeError, match="AMD GPUs only"):
+        lt.blocksparse_matmul(torch.randn(2, 8), torch.randn(8, 2, 2), torch.zeros(4, 2, dtype=torch.int32))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "leanffn.h")).read()
+    declared = set(re.findall(r"\b(lt_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(nat.EXPORTED_SYMBOLS), declared ^ set(nat.EXPORTED_SYMBOLS)
+    lib = nat.lib()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.lt_version().decode().startswith("libleanffn")
+
+
+def test_struct_layouts_match_header_sizes():
+    # pointer-sized and 4-byte members only: sizes are fixed by the C ABI on x86-64
+    assert ctypes.sizeof(nat.LtLinear) == 6 * 8 + 6 * 4
+    assert ctypes.sizeof(nat.LtLinearGrads) == 32
+    assert ctypes.sizeof(nat.LtFfnSaved) == 40
+    assert ctypes.sizeof(nat.LtFfnGrads) == 5 * 8 + 2 * 32
+    assert ctypes.sizeof(nat.LtFfnDesc) == 8 + 7 * 4 + 2 * 4 + 2 * 8 + 4 * 8 + 2 * ctypes.sizeof(nat.LtLinear) + 4
+
+
+def test_argument_errors_are_reported_not_crashed():
+    lib = nat.lib()
+    desc = nat.LtFfnDesc()  # all zero
+    assert lib.lt_ffn_forward_workspace_bytes(desc) == 0
+    status = lib.lt_ffn_forward(desc, None, None, nat.LtFfnSaved(), None, 0, None)
+    assert status == 1 and b"bad sizes" in lib.lt_last_error()
+    with pytest.raises(RuntimeError, match="lt_status 1"):
+        nat.check(status, "lt_ffn_forward")
