@@ -1,0 +1,155 @@
+"""LeanFFN fwd+bwd throughput on one MI355X: BASELINE config 3 (hidden 4096, intermediate 16384, GeGLU, bf16 weights, fp32
+residual stream, x [2, 2048, 4096]).  Prints one JSON line.
+
+    python bench.py --gpus 1 --steps 20 --warmup 5
+
+A step is one forward + backward of the module on a resident synthetic batch (parameter gradients produced, no optimizer).
+`roofline` is computed from HIP events recorded around every launch of the tiled bf16 MFMA GEMM kernel during the timed
+steps; `cpu_baseline` times the CPU oracle (tests' checker, not the product) on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "LeanFFN fwd+bwd tokens/s + MFMA util % at h4096 bf16; peak activation MB"
+PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk/CU x 2.4 GHz, dense
+
+
+def build_workload(torch, lt, batch, seq, hidden, inter, std, device):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(batch, seq, hidden, generator=g)
+    ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.i2h_proj.weight.copy_(torch.randn(2 * inter, hidden, generator=g) * std)
+        ffn.h2o_proj.weight.copy_(torch.randn(hidden, inter, generator=g) * std)
+        ffn.i2h_proj.bias.zero_()
+        ffn.h2o_proj.bias.zero_()
+    dy = torch.randn(batch, seq, hidden, generator=g)
+    ffn = ffn.to(device).to(torch.bfloat16)
+    return ffn, x.to(device).requires_grad_(True), dy.to(device)
+
+
+def cpu_baseline(torch, hidden, inter, std, sample_tokens, iters):
+    """the oracle's memory-lean autograd.Function (same save-set and recompute schedule as the reference's _LeanFFN) in fp32
+    on the host cores, on the first `sample_tokens` tokens of the workload"""
+    from oracle import ffn as offn
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(sample_tokens, hidden, generator=g)
+    p = offn.make_dense_params(hidden, inter, gated=True, std=std, generator=g, ln_eps=1e-5)
+    for t in p.tensors():
+        t.requires_grad_(True)
+    dy = torch.randn(sample_tokens, hidden, generator=g)
+    x.requires_grad_(True)
+    times = []
+    for i in range(iters + 1):
+        t0 = time.perf_counter()
+        y = offn.lean_ffn(x, p)
+        torch.autograd.grad(y, [x, *p.tensors()], dy)
+        times.append(time.perf_counter() - t0)
+    best = sorted(times[1:])[len(times[1:]) // 2]
+    return sample_tokens / best, best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no collectives and every box has one GPU (use --gpus 1)")
+
+    import torch
+
+    import lean_transformer_amd as lt
+    from lean_transformer_amd import _native as nat
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = torch.device("cuda:0")
+    batch, seq, hidden, inter, std = 2, 2048, 4096, 16384, 0.01
+    tokens = batch * seq
+    ffn, x, dy = build_workload(torch, lt, batch, seq, hidden, inter, std, device)
+    params = list(ffn.parameters())
+
+    def step():
+        y = ffn(x)
+        torch.autograd.grad(y, [x, *params], dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # peak activation memory of one fwd+bwd, relative to what is resident before it (parameters, x, dy)
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    y = ffn(x)
+    torch.cuda.synchronize()
+    saved_mb = (torch.cuda.memory_allocated() - base - y.numel() * y.element_size()) / 2**20
+    torch.autograd.grad(y, [x, *params], dy)
+    torch.cuda.synchronize()
+    peak_mb = (torch.cuda.max_memory_allocated() - base) / 2**20
+    del y
+
+    lib = nat.lib()
+    lib.lt_profile_reset()
+    lib.lt_profile_enable(1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.lt_profile_enable(0)
+    kernels = nat.profile_read()
+    lib.lt_profile_reset()
+
+    ms_per_step = elapsed / args.steps * 1e3
+    flops_per_step = 6.0 * tokens * hidden * (2 * inter + inter)
+    tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
+
+    gemm = [k for k in kernels if k[0].startswith("gemm_bf16")]
+    gemm_flops = sum(k[3] for k in gemm)
+    gemm_ms = sum(k[2] for k in gemm)
+    gemm_launches = sum(k[1] for k in gemm)
+    achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
+    kernel_table = [{"kernel": name, "launches": n, "avg_us": ms / n * 1e3,
+                     **({"tflops": fl / (ms * 1e-3) / 1e12} if fl > 0 else {}),
+                     **({"gbps": by / (ms * 1e-3) / 1e9} if by > 0 else {})} for name, n, ms, fl, by in kernels]
+
+    result = {
+        "metric": METRIC, "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "config3: LeanFFN dense GeGLU fwd+bwd, hidden 4096, intermediate 16384, x [2,2048,4096] fp32 "
+                               "residual stream, bf16 weights/activations, fp32 accumulation, dropout 0",
+                   "tokens": tokens, "hidden": hidden, "intermediate": inter},
+        "tflops": tflops, "mfma_util_pct": 100.0 * tflops / PEAK_BF16_TFLOPS,
+        "peak_activation_mb": peak_mb, "saved_activation_mb": saved_mb,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "gemm_bf16_kernel (tiled bf16 MFMA GEMM, all 6 launches per step)",
+                     "flops_per_launch": gemm_flops / max(gemm_launches, 1),
+                     "avg_launch_us": gemm_ms / max(gemm_launches, 1) * 1e3},
+        "kernels": kernel_table,
+    }
+    if not args.no_cpu_baseline:
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        sample = 256
+        value, sec = cpu_baseline(torch, hidden, inter, std, sample, iters=3)
+        result["cpu_baseline"] = {
+            "value": value, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle LeanFFNFunction (stock PyTorch fp32, reference save-set) on the first {sample} of {tokens} "
+                      f"tokens of the same config, median of 3 fwd+bwd after 1 warm-up, {sec:.2f} s each"}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -165,6 +165,23 @@ int lt_dropout_mask(int64_t tokens, int32_t hidden, float p, uint64_t seed, uint
 int lt_gemm(int32_t dtype, int64_t m, int64_t n, int64_t k, const void* a, int32_t a_kmajor, const void* b,
             int32_t b_kmajor, int32_t c_dtype, void* c, int32_t force_generic, void* stream);
 
+/* ---- per-kernel timing (no counterpart in the reference: measurement only) ----------------------------------------------
+ * While enabled, every kernel launch of the library is bracketed by two HIP events recorded on the launch stream.
+ * lt_profile_read waits for the recorded events and returns one aggregated entry per kernel tag: launches, total device
+ * milliseconds, and the algorithmic flops / bytes the launches stand for (0 where not applicable). */
+typedef struct lt_profile_entry {
+  char name[64];
+  int64_t launches;
+  double ms;
+  double flops;
+  double bytes;
+} lt_profile_entry;
+
+int lt_profile_enable(int32_t enable);
+int lt_profile_reset(void);
+/* fills at most max_entries entries, returns the number of distinct tags (negative lt_status on error) */
+int lt_profile_read(lt_profile_entry* entries, int32_t max_entries);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = (
     "lt_blocksparse_forward", "lt_blocksparse_backward",
     "lt_layernorm_forward", "lt_layernorm_backward_workspace_bytes", "lt_layernorm_backward",
     "lt_activation_forward", "lt_activation_backward", "lt_dropout_mask", "lt_gemm",
+    "lt_profile_enable", "lt_profile_reset", "lt_profile_read",
 )
 
 
@@ -48,6 +49,11 @@ class LtFfnDesc(ctypes.Structure):
         ("ln_weight", c_void_p), ("ln_bias", c_void_p), ("post_ln_weight", c_void_p), ("post_ln_bias", c_void_p),
         ("i2h", LtLinear), ("h2o", LtLinear),
     ]
+
+
+class LtProfileEntry(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 64), ("launches", c_int64), ("ms", ctypes.c_double), ("flops", ctypes.c_double),
+                ("bytes", ctypes.c_double)]
 
 
 class LtFfnSaved(ctypes.Structure):
@@ -93,6 +99,9 @@ def _declare(lib):
     lib.lt_dropout_mask.argtypes = [c_int64, c_int32, c_float, c_uint64, c_uint64, c_void_p, c_void_p]
     lib.lt_gemm.argtypes = [c_int32, c_int64, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_void_p,
                             c_int32, c_void_p]
+    lib.lt_profile_enable.argtypes = [c_int32]
+    lib.lt_profile_reset.argtypes = []
+    lib.lt_profile_read.argtypes = [POINTER(LtProfileEntry), c_int32]
     for name in EXPORTED_SYMBOLS:
         fn = getattr(lib, name)
         if fn.restype is ctypes.c_int:  # default restype: these return lt_status
@@ -155,3 +164,12 @@ def current_stream(device: torch.device) -> int:
 def workspace(nbytes: int, device: torch.device) -> torch.Tensor:
     """scratch memory from PyTorch's caching allocator (256-byte aligned like every fresh block of it)"""
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def profile_read():
+    """[(kernel tag, launches, total ms, algorithmic flops, algorithmic bytes)] recorded since the last lt_profile_reset"""
+    entries = (LtProfileEntry * 64)()
+    n = lib().lt_profile_read(entries, 64)
+    if n < 0:
+        check(-n, "lt_profile_read")
+    return [(e.name.decode(), e.launches, e.ms, e.flops, e.bytes) for e in entries[:min(n, 64)]]

@@ -275,6 +275,10 @@ int lt_ln_forward(int64_t T, int H, float eps, int x_dtype, const void* x, const
                   (!w || lt_aligned(w, 16)) && (!b || lt_aligned(b, 16)) && (!residual || lt_aligned(residual, 16));
   dim3 grid(blocks_for(T, 4)), block(256);
   DropoutParams d = drop ? *drop : make_dropout(0.f, 0, 0);
+  LtProfileScope scope(tail ? "layernorm_fwd_tail" : (y ? "layernorm_fwd" : "layernorm_stats"), 0.0,
+                       (double)T * H * (lt_dtype_size(x_dtype) + (y ? lt_dtype_size(y_dtype) : 0) +
+                                        (residual ? lt_dtype_size(res_dtype) : 0)) + (stats ? 8.0 * T : 0.0),
+                       stream);
 #define LT_LN_LAUNCH(TX, TY, TR, TAILV)                                                                              \
   hipLaunchKernelGGL((ln_fwd_kernel<TX, TY, TR, TAILV>), grid, block, 0, stream, T, H, eps, (const TX*)x, w, b, (TY*)y, \
                      stats, (const TR*)residual, d, vec)
@@ -313,6 +317,10 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
                "layernorm backward: workspace of %zu bytes needed", lt_ln_backward_workspace(T, H));
     partial = (float*)workspace;
   }
+  LtProfileScope scope("layernorm_bwd", 0.0,
+                       (double)T * H * (lt_dtype_size(x_dtype) + lt_dtype_size(dy_dtype) +
+                                        (dx ? lt_dtype_size(dx_dtype) : 0) + (residual_grad ? lt_dtype_size(dx_dtype) : 0)),
+                       stream);
   dim3 grid(nb), block(256);
 #define LT_LNB_LAUNCH(TX, TDY, TDX)                                                                                      \
   hipLaunchKernelGGL((ln_bwd_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
@@ -353,6 +361,7 @@ int lt_colsum(int64_t rows, int cols, int64_t ld, int dtype, const void* in, flo
   LT_REQUIRE(rows > 0 && cols > 0 && in && out, LT_ERR_BAD_ARG, "colsum: bad arguments");
   LT_REQUIRE(workspace && workspace_bytes >= lt_colsum_workspace(rows, cols), LT_ERR_WORKSPACE,
              "colsum: workspace of %zu bytes needed", lt_colsum_workspace(rows, cols));
+  LtProfileScope scope("colsum", 0.0, (double)rows * cols * lt_dtype_size(dtype), stream);
   const int slices = colsum_slices(rows);
   const int64_t rps = (rows + slices - 1) / slices;
   dim3 grid(blocks_for(cols, 64), slices), block(256);
@@ -369,6 +378,7 @@ int lt_colsum(int64_t rows, int cols, int64_t ld, int dtype, const void* in, flo
 
 int lt_act_forward(int64_t T, int64_t I, int gated, int act, int dtype, const void* pre, void* hid, hipStream_t stream) {
   LT_REQUIRE(T > 0 && I > 0 && pre && hid, LT_ERR_BAD_ARG, "activation: bad arguments");
+  LtProfileScope scope("activation_fwd", 0.0, (double)T * I * lt_dtype_size(dtype) * (gated ? 3 : 2), stream);
   dim3 grid(blocks_for(T * I, 256)), block(256);
   if (dtype == LT_F32)
     hipLaunchKernelGGL((act_fwd_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre, (float*)hid);
@@ -381,6 +391,7 @@ int lt_act_forward(int64_t T, int64_t I, int gated, int act, int dtype, const vo
 int lt_act_backward(int64_t T, int64_t I, int gated, int act, int dtype, const void* pre, const void* dhid, void* dpre,
                     hipStream_t stream) {
   LT_REQUIRE(T > 0 && I > 0 && pre && dhid && dpre, LT_ERR_BAD_ARG, "activation backward: bad arguments");
+  LtProfileScope scope("activation_bwd", 0.0, (double)T * I * lt_dtype_size(dtype) * (gated ? 5 : 3), stream);
   dim3 grid(blocks_for(T * I, 256)), block(256);
   if (dtype == LT_F32)
     hipLaunchKernelGGL((act_bwd_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre,
@@ -395,6 +406,7 @@ int lt_act_backward(int64_t T, int64_t I, int gated, int act, int dtype, const v
 int lt_dropout_cast(int64_t n, int in_dtype, const void* in, int out_dtype, void* out, const DropoutParams& drop,
                     hipStream_t stream) {
   LT_REQUIRE(n > 0 && in && out, LT_ERR_BAD_ARG, "dropout: bad arguments");
+  LtProfileScope scope("dropout_replay_cast", 0.0, (double)n * (lt_dtype_size(in_dtype) + lt_dtype_size(out_dtype)), stream);
   dim3 grid(blocks_for(n, 256)), block(256);
   const int key = (in_dtype == LT_BF16) * 2 + (out_dtype == LT_BF16);
   switch (key) {

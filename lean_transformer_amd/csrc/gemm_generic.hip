@@ -226,6 +226,15 @@ int lt_launch_gemm_generic(const GemmProblem& p, int kind, int dtype, int io_dty
   const int64_t tiles_n = (cols + (gated ? GBN / 2 : GBN) - 1) / (gated ? GBN / 2 : GBN);
   const int64_t tiles_m = (rows + GBM - 1) / GBM;
   LT_REQUIRE(tiles_m <= 65535, LT_ERR_UNSUPPORTED, "gemm: M=%lld exceeds the grid limit", (long long)p.M);
+  double flops = lt_gemm_flops(p, kind);
+  if (sp.mode == SPARSE_FWD || sp.mode == SPARSE_DX) {
+    flops = 2.0 * (double)p.M * (double)p.N * ((sp.mode == SPARSE_FWD ? sp.blocks_per_out : sp.blocks_per_in) * (double)sp.block +
+                                                (p.nseg > 1 ? (double)p.K[1] : 0.0));
+  } else if (sp.mode == SPARSE_DW) {
+    flops = 2.0 * (double)sp.tokens * (double)groups * sp.block * sp.block;
+  }
+  static const char* tags[4] = {"gemm_generic", "blocksparse_fwd_generic", "blocksparse_dx_generic", "blocksparse_dw_generic"};
+  LtProfileScope scope(tags[sp.mode], flops, 0.0, stream);
   dim3 grid((unsigned)tiles_n, (unsigned)tiles_m, (unsigned)groups);
   return dtype == LT_F32 ? launch_kind<float>(p, kind, io_dtype, grid, stream)
                          : launch_kind<bf16>(p, kind, io_dtype, grid, stream);

@@ -318,8 +318,24 @@ bool lt_gemm_mfma_supported(const GemmProblem& p, int kind) {
   return true;
 }
 
+static const char* mfma_tag(const GemmProblem& p, int kind) {
+  static const char* names[3][4] = {
+      {"gemm_bf16_nt_store", "gemm_bf16_nt_act_fwd", "gemm_bf16_nt_act_bwd", "gemm_bf16_nt_out"},
+      {"gemm_bf16_nn_store", "gemm_bf16_nn_act_fwd", "gemm_bf16_nn_act_bwd", "gemm_bf16_nn_out"},
+      {"gemm_bf16_tn_store", "gemm_bf16_tn_act_fwd", "gemm_bf16_tn_act_bwd", "gemm_bf16_tn_out"}};
+  const int layout = p.A[0].kmajor ? (p.B[0].kmajor ? 0 : 1) : 2;
+  return names[layout][kind];
+}
+
+double lt_gemm_flops(const GemmProblem& p, int kind) {
+  const double n = (kind == EPI_ACT_FWD && p.epi.gated) ? 2.0 * p.N : (double)p.N;
+  double k = (double)p.K[0] + (p.nseg > 1 ? (double)p.K[1] : 0.0);
+  return 2.0 * (double)p.M * n * k;
+}
+
 int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_t stream) {
   LT_REQUIRE(lt_gemm_mfma_supported(p, kind), LT_ERR_UNSUPPORTED, "tiled bf16 gemm does not take this problem");
+  LtProfileScope scope(mfma_tag(p, kind), lt_gemm_flops(p, kind), 0.0, stream);
   switch (kind) {
     case EPI_STORE: return launch_layout<EPI_STORE>(p, io_dtype, stream);
     case EPI_ACT_FWD: return launch_layout<EPI_ACT_FWD>(p, io_dtype, stream);

@@ -49,6 +49,23 @@ void lt_set_error(const char* fmt, ...);
     if (s_ != LT_OK) return s_; \
   } while (0)
 
+// ---------------------------------------------------------------------------------------------------------------------
+// optional per-kernel timing: a scope object brackets the launches issued while it lives with two events on `stream`
+// ---------------------------------------------------------------------------------------------------------------------
+bool lt_profile_active();
+void lt_profile_begin(const char* tag, double flops, double bytes, hipStream_t stream);
+void lt_profile_end(hipStream_t stream);
+struct LtProfileScope {
+  hipStream_t stream;
+  bool on;
+  LtProfileScope(const char* tag, double flops, double bytes, hipStream_t s) : stream(s), on(lt_profile_active()) {
+    if (on) lt_profile_begin(tag, flops, bytes, s);
+  }
+  ~LtProfileScope() {
+    if (on) lt_profile_end(stream);
+  }
+};
+
 static inline size_t lt_dtype_size(int dtype) { return dtype == LT_F32 ? 4 : 2; }
 static inline size_t lt_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 static inline bool lt_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
