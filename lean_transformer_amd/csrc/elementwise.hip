@@ -179,6 +179,102 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(int64_t T, int H, const TX*
   }
 }
 
+// Vectorised LayerNorm backward (hidden % 4 == 0, hidden <= 8192, 16-byte aligned rows), split in two so that neither half
+// has to keep per-column partial sums next to a cached row:
+//   ln_bwd_dx_kernel      one wavefront per row; dy and x of the row live in registers, the two row sums go through
+//                         shuffles, dx (+ residual gradient) is written with 16-byte stores
+//   ln_bwd_param_kernel   column-parallel: 64 lanes x 4 columns per workgroup and 4 row lanes walking a slice of rows;
+//                         writes one partial (dweight, dbias) row per slice, summed by colreduce_kernel
+template <typename TX, typename TDY, typename TDX>
+__global__ __launch_bounds__(256) void ln_bwd_dx_kernel(int64_t T, int H, const TX* __restrict__ x,
+                                                         const float* __restrict__ stats, const float* __restrict__ w,
+                                                         const TDY* __restrict__ dy, const TDX* __restrict__ residual_grad,
+                                                         TDX* __restrict__ dx) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= T) return;
+  const float mean = stats[row * 2], rstd = stats[row * 2 + 1];
+  const TX* xr = x + row * H;
+  const TDY* dyr = dy + row * H;
+  float xh[LN_MAXV][4], dxh[LN_MAXV][4];
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_MAXV; i++) {
+    const int c = (i * 64 + lane) * 4;
+    if (c < H) {
+      float wv[4];
+      load4(xr + c, xh[i]);
+      load4(dyr + c, dxh[i]);
+      load4(w + c, wv);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        xh[i][e] = (xh[i][e] - mean) * rstd;
+        dxh[i][e] *= wv[e];
+        s1 += dxh[i][e];
+        s2 += dxh[i][e] * xh[i][e];
+      }
+    }
+  }
+  const float inv_h = 1.0f / (float)H;
+  const float c1 = wave_sum(s1) * inv_h, c2 = wave_sum(s2) * inv_h;
+#pragma unroll
+  for (int i = 0; i < LN_MAXV; i++) {
+    const int c = (i * 64 + lane) * 4;
+    if (c < H) {
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) o[e] = rstd * (dxh[i][e] - c1 - xh[i][e] * c2);
+      if (residual_grad) {
+        float rv[4];
+        load4(residual_grad + row * H + c, rv);
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] += rv[e];
+      }
+      store4(dx + row * H + c, o);
+    }
+  }
+}
+
+template <typename TX, typename TDY>
+__global__ __launch_bounds__(256) void ln_bwd_param_kernel(int64_t T, int H, const TX* __restrict__ x,
+                                                            const float* __restrict__ stats, const TDY* __restrict__ dy,
+                                                            int64_t rows_per_slice, float* __restrict__ partial) {
+  __shared__ float red[4][64][8];
+  const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + cl) * 4;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice, r1 = min(T, r0 + rows_per_slice);
+  float pw[4] = {0.f, 0.f, 0.f, 0.f}, pb[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < H) {
+    for (int64_t r = r0 + rl; r < r1; r += 4) {
+      const float mean = stats[r * 2], rstd = stats[r * 2 + 1];
+      float xv[4], g[4];
+      load4(x + r * H + c, xv);
+      load4(dy + r * H + c, g);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        pw[e] += g[e] * ((xv[e] - mean) * rstd);
+        pb[e] += g[e];
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    red[rl][cl][e] = pw[e];
+    red[rl][cl][4 + e] = pb[e];
+  }
+  __syncthreads();
+  if (rl == 0 && c < H) {
+    float ow[4], ob[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      ow[e] = red[0][cl][e] + red[1][cl][e] + red[2][cl][e] + red[3][cl][e];
+      ob[e] = red[0][cl][4 + e] + red[1][cl][4 + e] + red[2][cl][4 + e] + red[3][cl][4 + e];
+    }
+    store4(partial + ((int64_t)blockIdx.y * 2) * H + c, ow);
+    store4(partial + ((int64_t)blockIdx.y * 2 + 1) * H + c, ob);
+  }
+}
+
 // out[c] = sum_r partial[r * stride + c], one thread per column (rows are few)
 __global__ void colreduce_kernel(int rows, int64_t stride, int cols, const float* __restrict__ partial,
                                  float* __restrict__ out) {
@@ -203,6 +299,40 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(int64_t rows, int c
   red[rl][cl] = s;
   __syncthreads();
   if (rl == 0 && c < cols) partial[(int64_t)blockIdx.y * cols + c] = red[0][cl] + red[1][cl] + red[2][cl] + red[3][cl];
+}
+
+// same with 8 consecutive columns per thread (16-byte loads for bf16): 32 column lanes x 8 row lanes per workgroup
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_partial8_kernel(int64_t rows, int cols, int64_t ld, const T* __restrict__ in,
+                                                               int64_t rows_per_slice, float* __restrict__ partial) {
+  __shared__ float red[8][32][9];
+  const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int c = (blockIdx.x * 32 + cl) * 8;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice, r1 = min(rows, r0 + rows_per_slice);
+  float s[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) s[e] = 0.f;
+  if (c < cols) {
+    for (int64_t r = r0 + rl; r < r1; r += 8) {
+      float v[8];
+      load8(in + r * ld + c, v);
+#pragma unroll
+      for (int e = 0; e < 8; e++) s[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) red[rl][cl][e] = s[e];
+  __syncthreads();
+  if (rl == 0 && c < cols) {
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      o[e] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; q++) o[e] += red[q][cl][e];
+    }
+    store8(partial + (int64_t)blockIdx.y * cols + c, o);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -301,8 +431,16 @@ int lt_ln_forward(int64_t T, int H, float eps, int x_dtype, const void* x, const
 }
 
 static int ln_bwd_blocks(int64_t T) { return (int)(T < 1024 ? T : 1024); }
+static int ln_bwd_slices(int64_t T) {
+  int64_t s = (T + 63) / 64;
+  return (int)(s < 1 ? 1 : (s > 128 ? 128 : s));
+}
 
-size_t lt_ln_backward_workspace(int64_t T, int H) { return (size_t)ln_bwd_blocks(T) * 2 * (size_t)H * sizeof(float); }
+// partial (dweight, dbias) rows: one pair per workgroup of the any-shape kernel or per row slice of the vectorised one
+size_t lt_ln_backward_workspace(int64_t T, int H) {
+  const int rows = ln_bwd_blocks(T) > ln_bwd_slices(T) ? ln_bwd_blocks(T) : ln_bwd_slices(T);
+  return (size_t)rows * 2 * (size_t)H * sizeof(float);
+}
 
 int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* stats, const float* w, int dy_dtype,
                    const void* dy, int dx_dtype, const void* residual_grad, void* dx, float* dweight, float* dbias,
@@ -310,7 +448,6 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   LT_REQUIRE(T > 0 && H > 0 && x && stats && w && dy, LT_ERR_BAD_ARG, "layernorm backward: bad arguments");
   LT_REQUIRE(H <= 256 * LNB_MAXC, LT_ERR_UNSUPPORTED, "layernorm backward: hidden size %d above %d", H, 256 * LNB_MAXC);
   LT_REQUIRE((dweight == nullptr) == (dbias == nullptr), LT_ERR_BAD_ARG, "layernorm backward: pass both dweight and dbias or neither");
-  const int nb = ln_bwd_blocks(T);
   float* partial = nullptr;
   if (dweight) {
     LT_REQUIRE(workspace && workspace_bytes >= lt_ln_backward_workspace(T, H), LT_ERR_WORKSPACE,
@@ -318,31 +455,73 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
     partial = (float*)workspace;
   }
   LtProfileScope scope("layernorm_bwd", 0.0,
-                       (double)T * H * (lt_dtype_size(x_dtype) + lt_dtype_size(dy_dtype) +
-                                        (dx ? lt_dtype_size(dx_dtype) : 0) + (residual_grad ? lt_dtype_size(dx_dtype) : 0)),
+                       (double)T * H * ((dx ? 1 : 0) + (dweight ? 1 : 0)) * (lt_dtype_size(x_dtype) + lt_dtype_size(dy_dtype)) +
+                           (double)T * H * ((dx ? lt_dtype_size(dx_dtype) : 0) + (dx && residual_grad ? lt_dtype_size(dx_dtype) : 0)),
                        stream);
-  dim3 grid(nb), block(256);
+  const int key = (x_dtype == LT_BF16) * 4 + (dy_dtype == LT_BF16) * 2 + (dx_dtype == LT_BF16);
+  const bool vec = (H & 3) == 0 && H <= 64 * 4 * LN_MAXV && lt_aligned(x, 16) && lt_aligned(dy, 16) && lt_aligned(w, 16) &&
+                   (!dx || lt_aligned(dx, 16)) && (!residual_grad || lt_aligned(residual_grad, 16)) &&
+                   (!partial || lt_aligned(partial, 16));
+  int partial_rows;
+  if (vec) {
+    if (dx) {
+      dim3 grid(blocks_for(T, 4)), block(256);
+#define LT_LNB_DX(TX, TDY, TDX)                                                                                         \
+  hipLaunchKernelGGL((ln_bwd_dx_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
+                     (const TDX*)residual_grad, (TDX*)dx)
+      switch (key) {
+        case 0: LT_LNB_DX(float, float, float); break;
+        case 1: LT_LNB_DX(float, float, bf16); break;
+        case 2: LT_LNB_DX(float, bf16, float); break;
+        case 3: LT_LNB_DX(float, bf16, bf16); break;
+        case 4: LT_LNB_DX(bf16, float, float); break;
+        case 5: LT_LNB_DX(bf16, float, bf16); break;
+        case 6: LT_LNB_DX(bf16, bf16, float); break;
+        default: LT_LNB_DX(bf16, bf16, bf16); break;
+      }
+#undef LT_LNB_DX
+      LT_LAUNCH_CHECK();
+    }
+    partial_rows = ln_bwd_slices(T);
+    if (partial) {
+      const int64_t rps = (T + partial_rows - 1) / partial_rows;
+      dim3 grid(blocks_for(H, 256), partial_rows), block(256);
+#define LT_LNB_PARAM(TX, TDY)                                                                                            \
+  hipLaunchKernelGGL((ln_bwd_param_kernel<TX, TDY>), grid, block, 0, stream, T, H, (const TX*)x, stats, (const TDY*)dy, rps, \
+                     partial)
+      switch (key >> 1) {
+        case 0: LT_LNB_PARAM(float, float); break;
+        case 1: LT_LNB_PARAM(float, bf16); break;
+        case 2: LT_LNB_PARAM(bf16, float); break;
+        default: LT_LNB_PARAM(bf16, bf16); break;
+      }
+#undef LT_LNB_PARAM
+      LT_LAUNCH_CHECK();
+    }
+  } else {
+    partial_rows = ln_bwd_blocks(T);
+    dim3 grid(partial_rows), block(256);
 #define LT_LNB_LAUNCH(TX, TDY, TDX)                                                                                      \
   hipLaunchKernelGGL((ln_bwd_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
                      (const TDX*)residual_grad, (TDX*)dx, partial)
-  const int key = (x_dtype == LT_BF16) * 4 + (dy_dtype == LT_BF16) * 2 + (dx_dtype == LT_BF16);
-  switch (key) {
-    case 0: LT_LNB_LAUNCH(float, float, float); break;
-    case 1: LT_LNB_LAUNCH(float, float, bf16); break;
-    case 2: LT_LNB_LAUNCH(float, bf16, float); break;
-    case 3: LT_LNB_LAUNCH(float, bf16, bf16); break;
-    case 4: LT_LNB_LAUNCH(bf16, float, float); break;
-    case 5: LT_LNB_LAUNCH(bf16, float, bf16); break;
-    case 6: LT_LNB_LAUNCH(bf16, bf16, float); break;
-    default: LT_LNB_LAUNCH(bf16, bf16, bf16); break;
-  }
+    switch (key) {
+      case 0: LT_LNB_LAUNCH(float, float, float); break;
+      case 1: LT_LNB_LAUNCH(float, float, bf16); break;
+      case 2: LT_LNB_LAUNCH(float, bf16, float); break;
+      case 3: LT_LNB_LAUNCH(float, bf16, bf16); break;
+      case 4: LT_LNB_LAUNCH(bf16, float, float); break;
+      case 5: LT_LNB_LAUNCH(bf16, float, bf16); break;
+      case 6: LT_LNB_LAUNCH(bf16, bf16, float); break;
+      default: LT_LNB_LAUNCH(bf16, bf16, bf16); break;
+    }
 #undef LT_LNB_LAUNCH
-  LT_LAUNCH_CHECK();
+    LT_LAUNCH_CHECK();
+  }
   if (dweight) {
-    // partial rows alternate (dweight, dbias): stride 2 * H between workgroups
-    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, nb, (int64_t)2 * H, H, partial,
-                       dweight);
-    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, nb, (int64_t)2 * H, H,
+    // partial rows alternate (dweight, dbias): stride 2 * H between them
+    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, partial_rows, (int64_t)2 * H, H,
+                       partial, dweight);
+    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, partial_rows, (int64_t)2 * H, H,
                        partial + H, dbias);
     LT_LAUNCH_CHECK();
   }
@@ -364,12 +543,20 @@ int lt_colsum(int64_t rows, int cols, int64_t ld, int dtype, const void* in, flo
   LtProfileScope scope("colsum", 0.0, (double)rows * cols * lt_dtype_size(dtype), stream);
   const int slices = colsum_slices(rows);
   const int64_t rps = (rows + slices - 1) / slices;
-  dim3 grid(blocks_for(cols, 64), slices), block(256);
   float* partial = (float*)workspace;
-  if (dtype == LT_F32)
-    hipLaunchKernelGGL((colsum_partial_kernel<float>), grid, block, 0, stream, rows, cols, ld, (const float*)in, rps, partial);
-  else
-    hipLaunchKernelGGL((colsum_partial_kernel<bf16>), grid, block, 0, stream, rows, cols, ld, (const bf16*)in, rps, partial);
+  if ((cols & 7) == 0 && (ld & 7) == 0 && lt_aligned(in, 16) && lt_aligned(partial, 16)) {
+    dim3 grid(blocks_for(cols, 256), slices), block(256);
+    if (dtype == LT_F32)
+      hipLaunchKernelGGL((colsum_partial8_kernel<float>), grid, block, 0, stream, rows, cols, ld, (const float*)in, rps, partial);
+    else
+      hipLaunchKernelGGL((colsum_partial8_kernel<bf16>), grid, block, 0, stream, rows, cols, ld, (const bf16*)in, rps, partial);
+  } else {
+    dim3 grid(blocks_for(cols, 64), slices), block(256);
+    if (dtype == LT_F32)
+      hipLaunchKernelGGL((colsum_partial_kernel<float>), grid, block, 0, stream, rows, cols, ld, (const float*)in, rps, partial);
+    else
+      hipLaunchKernelGGL((colsum_partial_kernel<bf16>), grid, block, 0, stream, rows, cols, ld, (const bf16*)in, rps, partial);
+  }
   hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(cols, 256)), dim3(256), 0, stream, slices, (int64_t)cols, cols,
                      partial, out);
   LT_LAUNCH_CHECK();
