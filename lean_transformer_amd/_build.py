@@ -11,8 +11,11 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libleanffn.so")
 SOURCES = ["ffn.hip", "elementwise.hip", "gemm_generic.hip", "gemm_mfma_bf16.hip", "profile.hip"]
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_{add,mul,fma}_f32 from scalar float code
+# -pragma-unroll-threshold: the fused GEMM epilogues index the accumulator registers from fully unrolled loops; left rolled
+# (the default threshold is too small for them) the accumulators would be demoted to scratch memory
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
+         "-packed-fp32-ops", "-mllvm", "-pragma-unroll-threshold=100000", "-Wno-unused-command-line-argument",
+         "-Wno-unknown-warning-option"]
 
 
 def _hipcc() -> str:

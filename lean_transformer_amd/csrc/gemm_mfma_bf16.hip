@@ -265,15 +265,20 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
 // A wavefront's copy instruction deposits the 64 lanes' 16-byte pieces at consecutive LDS addresses (lane i at base + 16 i),
 // so the swizzled LDS layouts are produced by choosing which global chunk each lane fetches.
 //
-// Tile 256 x 256, 4 wavefronts (2 x 2, 128 x 128 each), k-steps of 32, a ring of 4 LDS stages (each one array holding the
-// A and the B tile of a k-step, so that copies into one stage provably do not alias reads of another), k-loop unrolled by 4.
+// Tile 256 x 256, 4 wavefronts (2 x 2, 128 x 128 each), k-steps of 32, k-loop unrolled by 4.  Per operand, 64 KiB of LDS:
+//   mn-major  a ring of four [32 k][256] tiles, one k-step each; every row of a tile is 512 contiguous bytes in HBM.  The
+//             copy of k-step kt + 3 is issued during k-step kt.
+//   k-major   two [256][64 k] buffers, one block of two k-steps each, so that every row contributes a full 128-byte line
+//             to a copy (with 32 k per copy the L2 would see twice as many half-line requests).  The copy of block
+//             kt / 2 + 1 is issued during the even k-step kt.
+// Every LDS buffer is a separate array, so that copies into one provably do not alias reads of another.
 // Pipeline of k-step kt:
 //     matrix instructions on the first 16 k (fragments already in registers)
-//         interleaved with: LDS reads of the second 16 k, copies of k-step kt + 3 into the stage freed one barrier ago
+//         interleaved with: LDS reads of the second 16 k, the copies listed above
 //     wait until this wavefront's copies of k-step kt + 1 have landed and its LDS reads are done; workgroup barrier
 //     matrix instructions on the second 16 k
 //         interleaved with: LDS reads of the first 16 k of k-step kt + 1
-// Copies therefore have three k-steps to arrive, and no LDS read latency is exposed after the barrier.
+// so no LDS read latency is exposed after the barrier and copies have 1.5 (k-major) to 2.5 (mn-major) k-steps to land.
 // =====================================================================================================================
 __device__ const u32x4 lt_zero_chunk = {0u, 0u, 0u, 0u};  // source of the lanes past the end of a ragged reduction
 
@@ -292,9 +297,6 @@ template <int READS, int COPIES, int MFMAS, int G = 0> struct SchedInterleave3 {
   }
 };
 
-// k-major tile with 64-byte rows (32 k): four 16-byte chunks per row, four rows per 256-byte bank line
-__device__ __forceinline__ int swz_km32(int row) { return (row >> 2) & 3; }
-
 // wait until at most N of this wavefront's copies are in flight and all its LDS reads have returned, then barrier.
 // The wait is a real s_waitcnt instruction (not inline assembly) so that the compiler's own wait-count bookkeeping sees
 // that older copies have landed; the empty asm statements only keep it from moving LDS accesses across the barrier.
@@ -306,15 +308,76 @@ template <int N> __device__ __forceinline__ void wait_copies_and_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// Per-lane copy state of one operand: byte offsets of this wavefront's copy instructions relative to a wavefront-uniform
+// base that advances by `unit_bytes` per copy unit (k-major: a block of 64 k; mn-major: a k-step of 32 k).
+template <bool KM> struct DmaOperand {
+  static constexpr int LOADS = KM ? 8 : 4;  // copy instructions per wavefront per unit (32 or 16 KiB / 4 wavefronts / 1 KiB)
+  uint32_t off[LOADS];
+  int krow[LOADS];  // mn-major: k-row inside the k-step (for the ragged-reduction test)
+  const char* base;
+  int64_t unit_bytes;
+  int seg;
+
+  // row0: first row / column of the tile.  k-major only: rows are clamped below row_limit when row_limit > 0 (ragged M),
+  // and with pair_rows > 0 tile row r maps to the gated up-projection's weight rows (gate half, then linear half at
+  // + pair_rows), 64 of each per 128-row wavefront sub-tile.
+  __device__ __forceinline__ void setup(const GemmOperand& op, int s, int64_t row0, int64_t row_limit, int64_t pair_rows,
+                                        int wave, int lane) {
+    seg = s;
+    const int64_t ld = op.ld;
+    const char* ptr = reinterpret_cast<const char*>(op.ptr);
+#pragma unroll
+    for (int j = 0; j < LOADS; j++) {
+      const int q = (wave * LOADS + j) * 64 + lane;  // 16-byte slot of the LDS buffer this lane fills
+      if constexpr (KM) {
+        const int row = q >> 3, c = (q & 7) ^ swz_km(row);
+        int64_t g = row;
+        if (row_limit > 0) g = min(row0 + row, row_limit - 1) - row0;
+        if (pair_rows > 0) g = ((row & 127) >> 6) * pair_rows + (row >> 7) * 64 + (row & 63);
+        off[j] = (uint32_t)((g * ld + c * 8) * 2);
+        krow[j] = 0;
+      } else {
+        const int kr = q >> 5, c = (q & 31) ^ swz_mn(kr);
+        off[j] = (uint32_t)((kr * ld + c * 8) * 2);
+        krow[j] = kr;
+      }
+    }
+    base = KM ? ptr + row0 * ld * 2 : ptr + row0 * 2;
+    unit_bytes = KM ? 64 * 2 : DK * ld * 2;
+  }
+
+  // all copies of unit u (counted inside the k-segment) into `dst`; k_limit: reduction length for the ragged test
+  template <bool K_TAIL> __device__ __forceinline__ void issue(int u, bf16* dst, int wave, int64_t k_limit) const {
+#pragma unroll
+    for (int j = 0; j < LOADS; j++) {
+      const char* g = base + u * unit_bytes + off[j];
+      if constexpr (K_TAIL && !KM) {
+        if ((int64_t)u * DK + krow[j] >= k_limit) g = reinterpret_cast<const char*>(&lt_zero_chunk);
+      }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                       (__attribute__((address_space(3))) void*)(dst + (wave * LOADS + j) * 512), 16, 0, 0);
+    }
+  }
+};
+
 template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
-  constexpr int LOADS = 4;                       // copy instructions per wavefront per operand per k-step (16 KiB / 4 / 1 KiB)
-  constexpr int STAGE_ELEMS = (BM + BN) * DK;    // one stage: A tile then B tile
-  __shared__ __attribute__((aligned(1024))) bf16 stage0[STAGE_ELEMS];
-  __shared__ __attribute__((aligned(1024))) bf16 stage1[STAGE_ELEMS];
-  __shared__ __attribute__((aligned(1024))) bf16 stage2[STAGE_ELEMS];
-  __shared__ __attribute__((aligned(1024))) bf16 stage3[STAGE_ELEMS];
+  constexpr int KM_ELEMS = 256 * 64, MN_ELEMS = DK * 256;
+  // k-major operands use the two d buffers, mn-major ones the four s tiles; the unused set is never referenced and takes
+  // no LDS
+  __shared__ __attribute__((aligned(1024))) bf16 a_d0[KM_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 a_d1[KM_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 a_s0[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 a_s1[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 a_s2[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 a_s3[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 b_d0[KM_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 b_d1[KM_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 b_s0[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 b_s1[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 b_s2[MN_ELEMS];
+  __shared__ __attribute__((aligned(1024))) bf16 b_s3[MN_ELEMS];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -343,225 +406,239 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   const int kt_seg0 = (int)((p.K[0] + DK - 1) / DK);
   const int kt_total = kt_seg0 + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
 
-  // ---- per-lane byte offsets of this wavefront's copies, relative to a wavefront-uniform base that advances with k
-  uint32_t off_a[LOADS], off_b[LOADS];
-  int krow_a[LOADS], krow_b[LOADS];  // mn-major: k-row inside the k-step (for the ragged-reduction test)
-  const char* base_a = nullptr;
-  const char* base_b = nullptr;
-  int64_t step_a = 0, step_b = 0;  // bytes per k-step
-  auto setup_segment = [&](int seg) {
-    const int64_t lda = p.A[seg].ld, ldb = p.B[seg].ld;
-#pragma unroll
-    for (int j = 0; j < LOADS; j++) {
-      const int q = (wave * LOADS + j) * 64 + lane;  // 16-byte slot of the LDS tile this lane fills
-      if constexpr (A_KM) {
-        const int row = q >> 2, c = (q & 3) ^ swz_km32(row);
-        const int64_t gm = min(m0 + row, p.M - 1) - m0;
-        off_a[j] = (uint32_t)((gm * lda + c * 8) * 2);
-        krow_a[j] = 0;
-      } else {
-        const int kr = q / (BM / 8), c = (q % (BM / 8)) ^ swz_mn(kr);
-        off_a[j] = (uint32_t)((kr * lda + c * 8) * 2);
-        krow_a[j] = kr;
-      }
-      if constexpr (B_KM) {
-        const int row = q >> 2, c = (q & 3) ^ swz_km32(row);
-        int64_t gn;
-        if (gated) {
-          const int rr = row % WTN;
-          gn = (rr / (WTN / 2)) * p.N + (row / WTN) * (WTN / 2) + rr % (WTN / 2);
-        } else {
-          gn = row;
-        }
-        off_b[j] = (uint32_t)((gn * ldb + c * 8) * 2);
-        krow_b[j] = 0;
-      } else {
-        const int kr = q / (BN / 8), c = (q % (BN / 8)) ^ swz_mn(kr);
-        off_b[j] = (uint32_t)((kr * ldb + c * 8) * 2);
-        krow_b[j] = kr;
-      }
-    }
-    const char* a = reinterpret_cast<const char*>(p.A[seg].ptr);
-    const char* b = reinterpret_cast<const char*>(p.B[seg].ptr);
-    base_a = A_KM ? a + m0 * lda * 2 : a + m0 * 2;
-    base_b = B_KM ? b + n0 * ldb * 2 : b + n0 * 2;
-    step_a = A_KM ? DK * 2 : DK * lda * 2;
-    step_b = B_KM ? DK * 2 : DK * ldb * 2;
+  // ---- buffer of k-step position I (k-step index mod 4) and copy targets, selected at compile time
+  auto a_buf = [&](auto I) -> bf16* {
+    constexpr int i = decltype(I)::value & 3;
+    if constexpr (A_KM) return (i & 2) ? a_d1 : a_d0;
+    else return i == 0 ? a_s0 : i == 1 ? a_s1 : i == 2 ? a_s2 : a_s3;
   };
-  setup_segment(0);
-  int copy_seg = 0;  // segment the offsets above belong to
+  auto b_buf = [&](auto I) -> bf16* {
+    constexpr int i = decltype(I)::value & 3;
+    if constexpr (B_KM) return (i & 2) ? b_d1 : b_d0;
+    else return i == 0 ? b_s0 : i == 1 ? b_s1 : i == 2 ? b_s2 : b_s3;
+  };
 
-  // all copies of k-step kt (2 * LOADS instructions) into stage `st`
-  auto issue_copies = [&](auto steady, int kt, bf16* st) {
-    int seg = copy_seg;
-    if constexpr (!decltype(steady)::value) {  // the steady loop never crosses a segment boundary
-      seg = kt >= kt_seg0;
-      if (seg != copy_seg) {
-        setup_segment(seg);
-        copy_seg = seg;
-      }
+  DmaOperand<A_KM> ca;
+  DmaOperand<B_KM> cb;
+  auto setup_a = [&](int seg) { ca.setup(p.A[seg], seg, m0, A_KM ? p.M : 0, 0, wave, lane); };
+  auto setup_b = [&](int seg) { cb.setup(p.B[seg], seg, n0, 0, (B_KM && gated) ? p.N : 0, wave, lane); };
+  setup_a(0);
+  setup_b(0);
+  // copies of the unit that holds k-step t (a block for k-major operands) into the buffer of position I
+  auto copy_a = [&](auto steady, auto I, int t) {
+    int seg = ca.seg;
+    if constexpr (!decltype(steady)::value) {  // the steady loop never crosses a k-segment boundary
+      seg = t >= kt_seg0;
+      if (seg != ca.seg) setup_a(seg);
     }
-    const int ks = seg ? kt - kt_seg0 : kt;
-#pragma unroll
-    for (int j = 0; j < LOADS; j++) {
-      const char* ga = base_a + ks * step_a + off_a[j];
-      const char* gb = base_b + ks * step_b + off_b[j];
-      if constexpr (K_TAIL) {
-        const int64_t K = p.K[seg];
-        if (!A_KM && (int64_t)ks * DK + krow_a[j] >= K) ga = reinterpret_cast<const char*>(&lt_zero_chunk);
-        if (!B_KM && (int64_t)ks * DK + krow_b[j] >= K) gb = reinterpret_cast<const char*>(&lt_zero_chunk);
-      }
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ga,
-                                       (__attribute__((address_space(3))) void*)(st + (wave * LOADS + j) * 512), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gb,
-                                       (__attribute__((address_space(3))) void*)(st + BM * DK + (wave * LOADS + j) * 512), 16,
-                                       0, 0);
-    }
+    const int ks = seg ? t - kt_seg0 : t;
+    ca.template issue<K_TAIL>(A_KM ? ks >> 1 : ks, a_buf(I), wave, p.K[seg]);
   };
-  auto frag_km = [&](const bf16* tile, int base, int kk) -> bf16x8 {
+  auto copy_b = [&](auto steady, auto I, int t) {
+    int seg = cb.seg;
+    if constexpr (!decltype(steady)::value) {
+      seg = t >= kt_seg0;
+      if (seg != cb.seg) setup_b(seg);
+    }
+    const int ks = seg ? t - kt_seg0 : t;
+    cb.template issue<K_TAIL>(B_KM ? ks >> 1 : ks, b_buf(I), wave, p.K[seg]);
+  };
+
+  // ---- MFMA operand fragments: 8 k values of row / column lane % 32 of a 32-wide block
+  auto frag_km = [&](const bf16* buf, int base, int kk, int half) -> bf16x8 {
     const int row = base + (lane & 31);
-    const int c = kk * 2 + (lane >> 5);
-    return *reinterpret_cast<const bf16x8*>(&tile[(row * 4 + (c ^ swz_km32(row))) * 8]);
+    const int c = half * 4 + kk * 2 + (lane >> 5);
+    return *reinterpret_cast<const bf16x8*>(&buf[(row * 8 + (c ^ swz_km(row))) * 8]);
   };
-  auto frag_mn = [&](const bf16* tile, int cols, int base, int kk) -> bf16x8 {
+  auto frag_mn = [&](const bf16* tile, int base, int kk) -> bf16x8 {
     union { bf16x8 v; s16x4 h[2]; } u;
     const int i16 = lane & 15;
     const int col = base + ((lane >> 4) & 1) * 16 + 4 * (i16 & 3);
 #pragma unroll
     for (int s = 0; s < 2; s++) {
       const int kr = kk * 16 + 8 * (lane >> 5) + 4 * s + (i16 >> 2);
-      const bf16* src = &tile[kr * cols + ((((col >> 3) ^ swz_mn(kr)) << 3) | (col & 7))];
+      const bf16* src = &tile[kr * 256 + ((((col >> 3) ^ swz_mn(kr)) << 3) | (col & 7))];
       u.h[s] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(src));
     }
     return u.v;
   };
-  auto load_frags = [&](const bf16* st, int kk, bf16x8 (&a)[FM], bf16x8 (&b)[FN]) {
+  auto load_frags = [&](auto I, int kk, bf16x8 (&a)[FM], bf16x8 (&b)[FN]) {
+    constexpr int half = decltype(I)::value & 1;
+    const bf16* ta = a_buf(I);
+    const bf16* tb = b_buf(I);
 #pragma unroll
     for (int i = 0; i < FM; i++) {
-      if constexpr (A_KM) a[i] = frag_km(st, wm * WTM + i * 32, kk);
-      else a[i] = frag_mn(st, BM, wm * WTM + i * 32, kk);
+      if constexpr (A_KM) a[i] = frag_km(ta, wm * WTM + i * 32, kk, half);
+      else a[i] = frag_mn(ta, wm * WTM + i * 32, kk);
     }
 #pragma unroll
     for (int j = 0; j < FN; j++) {
-      if constexpr (B_KM) b[j] = frag_km(st + BM * DK, wn * WTN + j * 32, kk);
-      else b[j] = frag_mn(st + BM * DK, BN, wn * WTN + j * 32, kk);
+      if constexpr (B_KM) b[j] = frag_km(tb, wn * WTN + j * 32, kk, half);
+      else b[j] = frag_mn(tb, wn * WTN + j * 32, kk);
     }
   };
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);
+  constexpr int N_MN = (A_KM ? 0 : 4) + (B_KM ? 0 : 4);  // copy instructions per k-step for the mn-major operands
+  constexpr int N_KM = (A_KM ? 8 : 0) + (B_KM ? 8 : 0);  // copy instructions per block for the k-major operands
 
   bf16x8 af[2][FM], bfr[2][FN];  // [0]: first 16 k of the current k-step, [1]: second 16 k
 
   // A k-step is issued as two halves so that the loop body can start at the barrier:
-  //   first_half(kt)   LDS reads of the second 16 k of k-step kt (stage `cur`), copies of k-step kt + 3 into `cpy`,
-  //                    matrix instructions on the first 16 k
-  //   second_half(kt)  wait for the copies of k-step kt + 1 + barrier, LDS reads of the first 16 k of k-step kt + 1 (stage
-  //                    `nxt`), matrix instructions on the second 16 k
-  // steady == true: straight-line code for k-steps far enough from the end of their k-segment.
-  auto first_half = [&](auto steady, int kt, const bf16* cur, bf16* cpy) {
+  //   first_half(t)   LDS reads of the second 16 k of k-step t, the copies due at t, matrix instructions on the first 16 k
+  //   second_half(t)  wait for the copies k-step t + 1 needs + barrier, LDS reads of the first 16 k of k-step t + 1,
+  //                   matrix instructions on the second 16 k
+  // I = t mod 4 at compile time.  steady == true: straight-line code, valid while every copy it issues exists and stays
+  // inside the current k-segment.
+  auto first_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
-    load_frags(cur, 1, af[1], bfr[1]);
-    if (STEADY || kt + 3 < kt_total) issue_copies(steady, kt + 3, cpy);
+    constexpr int i = decltype(I)::value & 3;
+    load_frags(I, 1, af[1], bfr[1]);
+    if (STEADY || t + 3 < kt_total) {  // mn-major: k-step t + 3 into the tile freed by the last barrier
+      if constexpr (!A_KM) copy_a(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+      if constexpr (!B_KM) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+    }
+    if constexpr ((i & 1) == 0 && N_KM > 0) {  // k-major: the block of k-steps t + 2, t + 3 into the other buffer
+      if (STEADY || t + 2 < kt_total) {
+        if constexpr (A_KM) copy_a(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
+        if constexpr (B_KM) copy_b(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
+      }
+    }
 #pragma unroll
-    for (int i = 0; i < FM; i++)
+    for (int x = 0; x < FM; x++)
 #pragma unroll
-      for (int j = 0; j < FN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][i], bfr[0][j], acc[i][j], 0, 0, 0);
-    SchedInterleave3<FRAG_READS, 2 * LOADS, FM * FN>::run();
+      for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][x], bfr[0][y], acc[x][y], 0, 0, 0);
+    SchedInterleave3<FRAG_READS, N_MN + ((i & 1) == 0 ? N_KM : 0), FM * FN>::run();
   };
-  auto second_half = [&](auto steady, int kt, const bf16* nxt) {
+  auto second_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
-    const int remaining = kt_total - 1 - kt;  // k-steps after this one
-    // copies still allowed in flight: those of k-steps kt + 2 and kt + 3 (issued after the ones of kt + 1)
-    if (STEADY || remaining >= 3) wait_copies_and_barrier<4 * LOADS>();
-    else if (remaining == 2) wait_copies_and_barrier<2 * LOADS>();
+    constexpr int i = decltype(I)::value & 3;
+    // Copies complete in issue order.  Issued after the ones k-step t + 1 needs, and therefore allowed in flight:
+    //   t even: mn(t + 2), mn(t + 3), km(block of t + 2)      t odd: mn(t + 3) only (the block of t + 1 must have landed)
+    constexpr int IN_FLIGHT = N_KM == 0 ? 2 * N_MN : ((i & 1) == 0 ? 2 * N_MN + N_KM : N_MN);
+    if constexpr (STEADY) wait_copies_and_barrier<IN_FLIGHT>();
     else wait_copies_and_barrier<0>();
-    if (STEADY || remaining >= 1) load_frags(nxt, 0, af[0], bfr[0]);
+    if (STEADY || t + 1 < kt_total) load_frags(std::integral_constant<int, (i + 1) & 3>{}, 0, af[0], bfr[0]);
 #pragma unroll
-    for (int i = 0; i < FM; i++)
+    for (int x = 0; x < FM; x++)
 #pragma unroll
-      for (int j = 0; j < FN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][i], bfr[1][j], acc[i][j], 0, 0, 0);
+      for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][x], bfr[1][y], acc[x][y], 0, 0, 0);
     SchedInterleave3<FRAG_READS, 0, FM * FN>::run();
   };
   using Steady = std::integral_constant<bool, true>;
   using Ragged = std::integral_constant<bool, false>;
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using P2 = std::integral_constant<int, 2>;
+  using P3 = std::integral_constant<int, 3>;
 
-  // ---- prologue: first three k-steps in flight, the first one landed, first half of k-step 0 issued
-  issue_copies(Ragged{}, 0, stage0);
-  if (kt_total > 1) issue_copies(Ragged{}, 1, stage1);
-  if (kt_total > 2) issue_copies(Ragged{}, 2, stage2);
-  if (kt_total > 2) wait_copies_and_barrier<4 * LOADS>();
-  else if (kt_total == 2) wait_copies_and_barrier<2 * LOADS>();
-  else wait_copies_and_barrier<0>();
-  load_frags(stage0, 0, af[0], bfr[0]);
-  first_half(Ragged{}, 0, stage0, stage3);
+  // ---- prologue: k-steps 0..2 (k-major: block 0) in flight and landed, first half of k-step 0 issued
+  if constexpr (A_KM) copy_a(Ragged{}, P0{}, 0);
+  if constexpr (B_KM) copy_b(Ragged{}, P0{}, 0);
+  if constexpr (!A_KM) copy_a(Ragged{}, P0{}, 0);
+  if constexpr (!B_KM) copy_b(Ragged{}, P0{}, 0);
+  if (kt_total > 1) {
+    if constexpr (!A_KM) copy_a(Ragged{}, P1{}, 1);
+    if constexpr (!B_KM) copy_b(Ragged{}, P1{}, 1);
+  }
+  if (kt_total > 2) {
+    if constexpr (!A_KM) copy_a(Ragged{}, P2{}, 2);
+    if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2);
+  }
+  wait_copies_and_barrier<0>();
+  load_frags(P0{}, 0, af[0], bfr[0]);
+  first_half(Ragged{}, P0{}, 0);
 
   // loop body i of a group of four: second half of k-step kt + i, first half of k-step kt + i + 1
   int kt = 0;
   for (;;) {
-    // copies issued by the steady loop (k-steps up to kt + 7) must stay inside the k-segment the offsets are set up for
-    const int bound = (copy_seg == 0 && p.nseg > 1) ? kt_seg0 : kt_total;
-    for (; kt + 7 < bound; kt += 4) {
-      second_half(Steady{}, kt, stage1);
-      first_half(Steady{}, kt + 1, stage1, stage0);
-      second_half(Steady{}, kt + 1, stage2);
-      first_half(Steady{}, kt + 2, stage2, stage1);
-      second_half(Steady{}, kt + 2, stage3);
-      first_half(Steady{}, kt + 3, stage3, stage2);
-      second_half(Steady{}, kt + 3, stage0);
-      first_half(Steady{}, kt + 4, stage0, stage3);
+    // copies issued by the steady loop reach k-step kt + 7: they must exist and lie in the k-segment both operands' copy
+    // offsets are set up for
+    const int bound = (ca.seg == 0 && p.nseg > 1) ? kt_seg0 : kt_total;
+    if (ca.seg == cb.seg) {
+      for (; kt + 7 < bound; kt += 4) {
+        second_half(Steady{}, P0{}, kt);
+        first_half(Steady{}, P1{}, kt + 1);
+        second_half(Steady{}, P1{}, kt + 1);
+        first_half(Steady{}, P2{}, kt + 2);
+        second_half(Steady{}, P2{}, kt + 2);
+        first_half(Steady{}, P3{}, kt + 3);
+        second_half(Steady{}, P3{}, kt + 3);
+        first_half(Steady{}, P0{}, kt + 4);
+      }
     }
     if (kt >= kt_total) break;
-    second_half(Ragged{}, kt, stage1);
-    if (kt + 1 < kt_total) { first_half(Ragged{}, kt + 1, stage1, stage0); second_half(Ragged{}, kt + 1, stage2); }
-    if (kt + 2 < kt_total) { first_half(Ragged{}, kt + 2, stage2, stage1); second_half(Ragged{}, kt + 2, stage3); }
-    if (kt + 3 < kt_total) { first_half(Ragged{}, kt + 3, stage3, stage2); second_half(Ragged{}, kt + 3, stage0); }
-    if (kt + 4 < kt_total) first_half(Ragged{}, kt + 4, stage0, stage3);
+    second_half(Ragged{}, P0{}, kt);
+    if (kt + 1 < kt_total) { first_half(Ragged{}, P1{}, kt + 1); second_half(Ragged{}, P1{}, kt + 1); }
+    if (kt + 2 < kt_total) { first_half(Ragged{}, P2{}, kt + 2); second_half(Ragged{}, P2{}, kt + 2); }
+    if (kt + 3 < kt_total) { first_half(Ragged{}, P3{}, kt + 3); second_half(Ragged{}, P3{}, kt + 3); }
+    if (kt + 4 < kt_total) first_half(Ragged{}, P0{}, kt + 4);
     kt += 4;
     if (kt >= kt_total) break;
   }
-  __syncthreads();  // every wavefront is done with the stages: they become epilogue staging space
+  __syncthreads();  // every wavefront is done with the buffers: they become epilogue staging space
 
-  // ---- epilogue: as in the register-staged kernel; each wavefront stages its strips in a stage array of its own
-  constexpr int STAGE_LD = WTN + 8;
-  static_assert(32 * STAGE_LD * 4 <= STAGE_ELEMS * 2, "a 32-row strip must fit one stage array");
-  float* stage = reinterpret_cast<float*>(wave == 0 ? stage0 : wave == 1 ? stage1 : wave == 2 ? stage2 : stage3);
+  // ---- epilogue.  The accumulators of a 32 x 32 block sit column-per-lane (register r = row 8 * (r / 4) + 4 * (lane / 32)
+  //      + r % 4, column lane % 32).  Each wavefront transposes one 32-row strip of its sub-tile at a time through an LDS
+  //      buffer of its own (32 x 128 floats = 16 KiB, the size of the smallest buffer) and reads it back row-major, 8
+  //      consecutive columns per lane, so that the fused epilogue reads and writes HBM in 16-byte pieces of contiguous rows.
+  //      Staged column c of row r sits at c ^ 32 when bit 2 of r is set: the two half-waves of a transposing write (rows
+  //      r and r + 4, same columns) then hit different banks without padding the rows.
+  float* stage = reinterpret_cast<float*>(wave == 0   ? (A_KM ? a_d0 : a_s0)
+                                          : wave == 1 ? (A_KM ? a_d1 : a_s1)
+                                          : wave == 2 ? (B_KM ? b_d0 : b_s0)
+                                                      : (B_KM ? b_d1 : b_s1));
+  static_assert(32 * WTN * 4 <= MN_ELEMS * 2, "a 32-row strip must fit the smallest buffer");
+  auto staged = [&](int row, int col) -> float* { return &stage[row * WTN + (col ^ (((row >> 2) & 1) << 5))]; };
   const bool pair = (KIND == EPI_ACT_FWD) && gated;
 #pragma unroll
   for (int i = 0; i < FM; i++) {
 #pragma unroll
     for (int j = 0; j < FN; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++)
-        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * STAGE_LD + j * 32 + (lane & 31)] = acc[i][j][r];
+      for (int r = 0; r < 16; r++) *staged(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), j * 32 + (lane & 31)) = acc[i][j][r];
     __builtin_amdgcn_wave_barrier();
     const int64_t mrow0 = m0 + wm * WTM + i * 32;
     if (pair) {
+      // columns [0, WTN/2) of the sub-tile are gate columns, [WTN/2, WTN) the matching linear columns
       constexpr int LANES_PER_ROW = WTN / 2 / 8, ROWS_PER_IT = 64 / LANES_PER_ROW;
       for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
         const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW, c = (lane % LANES_PER_ROW) * 8;
         const int64_t m = mrow0 + row;
         float vg[8], vl[8];
+        const float* sg = staged(row, c);
+        const float* sl = staged(row, WTN / 2 + c);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-          vg[e] = stage[row * STAGE_LD + c + e];
-          vl[e] = stage[row * STAGE_LD + WTN / 2 + c + e];
+          vg[e] = sg[e];
+          vl[e] = sl[e];
         }
         if (m < p.M) epi_act_fwd_gated8(p.epi, m, n0 + wn * (WTN / 2) + c, vg, vl);
       }
     } else {
-      constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW;
-      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
-        const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW, c = (lane % LANES_PER_ROW) * 8;
+      constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+      const int c = (lane % LANES_PER_ROW) * 8;
+      const int64_t n = n0 + wn * WTN + c;
+      const int64_t mlane = mrow0 + lane / LANES_PER_ROW;  // this lane's row in iteration 0
+      // global reads of the epilogue run two iterations ahead of their use
+      EpiLoad l0 = epi_load8<KIND, TX>(p.epi, mlane, n, mlane < p.M);
+      EpiLoad l1 = epi_load8<KIND, TX>(p.epi, mlane + ROWS_PER_IT, n, mlane + ROWS_PER_IT < p.M);
+      for (int it = 0; it < NIT; it++) {
+        const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
         const int64_t m = mrow0 + row;
-        const int64_t n = n0 + wn * WTN + c;
+        const int64_t m2 = m + 2 * ROWS_PER_IT;
+        const EpiLoad l2 = epi_load8<KIND, TX>(p.epi, m2, n, it + 2 < NIT && m2 < p.M);
         float v[8];
+        const float* sv = staged(row, c);
 #pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = stage[row * STAGE_LD + c + e];
+        for (int e = 0; e < 8; e++) v[e] = sv[e];
         if (m < p.M) {
           if constexpr (KIND == EPI_STORE) epi_store8(p.epi, m, n, v);
           else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(p.epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8(p.epi, m, n, v);
-          else epi_out8<TX>(p.epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(p.epi, m, n, v, l0);
+          else epi_out8_loaded<TX>(p.epi, m, n, v, l0);
         }
+        l0 = l1;
+        l1 = l2;
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -623,9 +700,13 @@ bool dma_offsets_fit(const GemmProblem& p, int kind) {
 int g_mfma_variant = 0;  // 0: choose; 1: register-staged kernel; 2: copy-based kernel (tests and benchmarks)
 
 template <bool A_KM, bool B_KM, int KIND> int launch_tile(const GemmProblem& p, int io_dtype, hipStream_t stream) {
-  bool k_tail = false;
-  for (int s = 0; s < p.nseg; s++) k_tail = k_tail || (p.K[s] % DK != 0);
-  const bool dma_ok = dma_offsets_fit(p, KIND) && !(k_tail && KIND == EPI_OUT && io_dtype == LT_BF16);
+  bool k_tail = false, k_blocks = true;
+  for (int s = 0; s < p.nseg; s++) {
+    k_tail = k_tail || (p.K[s] % DK != 0);
+    k_blocks = k_blocks && (p.K[s] % 64 == 0);  // k-major operands are copied in whole blocks of 64 k
+  }
+  const bool dma_ok = dma_offsets_fit(p, KIND) && !(k_tail && KIND == EPI_OUT && io_dtype == LT_BF16) &&
+                      ((!A_KM && !B_KM) || k_blocks);
   if (g_mfma_variant != 1 && dma_ok) return launch_dma<A_KM, B_KM, KIND>(p, io_dtype, stream);
   return launch_cfg<256, 256, 2, 2, A_KM, B_KM, KIND>(p, io_dtype, stream);
 }

@@ -227,6 +227,100 @@ template <typename TX> __device__ __forceinline__ void epi_out8(const EpiParams&
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
+// Epilogues that READ global memory (the pre-activation in EPI_ACT_BWD, the residual in EPI_OUT) are split into a load
+// step and a compute/store step, so that the tiled kernel can keep the loads of later rows in flight while it works on
+// the current ones (a workgroup owns a whole compute unit there: nobody else hides its memory latency).
+// ---------------------------------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int lt_u32x4;
+struct EpiLoad {
+  lt_u32x4 a, b;  // EPI_ACT_BWD: 8 gate and 8 linear pre-activations (bf16); EPI_OUT: 8 residual values (fp32: a|b, bf16: a)
+};
+
+template <int KIND, typename TX>
+__device__ __forceinline__ EpiLoad epi_load8(const EpiParams& e, int64_t m, int64_t n, bool valid) {
+  EpiLoad l;
+  l.a = lt_u32x4{0u, 0u, 0u, 0u};
+  l.b = l.a;
+  if (!valid) return l;
+  if constexpr (KIND == EPI_ACT_BWD) {
+    const bf16* pre = reinterpret_cast<const bf16*>(e.pre) + m * e.ld_pre + n;
+    l.a = *reinterpret_cast<const lt_u32x4*>(pre);
+    if (e.gated) l.b = *reinterpret_cast<const lt_u32x4*>(pre + e.inter);
+  } else if constexpr (KIND == EPI_OUT) {
+    if (e.x) {
+      const TX* x = reinterpret_cast<const TX*>(e.x) + m * e.ldy + n;
+      l.a = *reinterpret_cast<const lt_u32x4*>(x);
+      if constexpr (sizeof(TX) == 4) l.b = *reinterpret_cast<const lt_u32x4*>(x + 4);
+    }
+  }
+  return l;
+}
+
+__device__ __forceinline__ void unpack_bf16x8(const lt_u32x4& raw, float (&v)[8]) {
+  union { lt_u32x4 u; bf16 h[8]; } t;
+  t.u = raw;
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = (float)t.h[i];
+}
+
+__device__ __forceinline__ void epi_act_bwd8_loaded(const EpiParams& e, int64_t m, int64_t n, const float (&dh)[8],
+                                                    const EpiLoad& l) {
+  bf16* dpre = reinterpret_cast<bf16*>(e.dpre) + m * e.ld_pre + n;
+  float pg[8], a[8], da[8], o[8];
+  unpack_bf16x8(l.a, pg);
+#pragma unroll
+  for (int i = 0; i < 8; i++) act_eval<false>(e.act, pg[i], a[i], da[i]);
+  if (e.gated) {
+    float pl[8];
+    unpack_bf16x8(l.b, pl);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * pl[i] * da[i];
+    store8(dpre, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * a[i];
+    store8(dpre + e.inter, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] *= pl[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * da[i];
+    store8(dpre, o);
+  }
+  if (e.hid) store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, a);
+}
+
+template <typename TX>
+__device__ __forceinline__ void epi_out8_loaded(const EpiParams& e, int64_t m, int64_t n, float (&v)[8], const EpiLoad& l) {
+  add_bias8(e.bias, n, v);
+  const int64_t idx = m * e.ldy + n;
+  if (e.drop.p > 0.f) {
+    bool k0[4], k1[4];
+    dropout_keep4(e.drop, idx, k0);
+    dropout_keep4(e.drop, idx + 4, k1);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[i] = k0[i] ? v[i] * e.drop.scale : 0.f;
+      v[i + 4] = k1[i] ? v[i + 4] * e.drop.scale : 0.f;
+    }
+  }
+  if (e.x) {
+    float r[8];
+    if constexpr (sizeof(TX) == 4) {
+      union { lt_u32x4 u[2]; float f[8]; } t;
+      t.u[0] = l.a;
+      t.u[1] = l.b;
+#pragma unroll
+      for (int i = 0; i < 8; i++) r[i] = t.f[i];
+    } else {
+      unpack_bf16x8(l.a, r);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] += r[i];
+  }
+  store8(reinterpret_cast<TX*>(e.y) + idx, v);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
 // launchers (defined in gemm_generic.hip / gemm_mfma_bf16.hip)
 // ---------------------------------------------------------------------------------------------------------------------
 // any shape, fp32 or bf16 operands (dtype), fp32 MFMA arithmetic.  io_dtype: dtype of x / y for EPI_OUT.

@@ -330,6 +330,62 @@ def test_config3_bf16_full_size_headline():
     _full_size_checks(ffn, x, dy, 0.0)
 
 
+@pytest.mark.parametrize("stretch", [True, False])
+def test_config4_pixelfly_bf16_full_size(stretch):
+    """BASELINE config 4: config 3's shape with PixelFly block-sparse projections (64 x 64 blocks, 7 of 64 blocks per block
+    row: up-projection K/A = 7/56, down-projection 28/7) plus a rank-128 low-rank term, bf16"""
+    g = torch.Generator().manual_seed(0)
+    hidden, inter, rank = 4096, 16384, 128
+    layout = f"pixelfly(block_size=64, stretch={stretch})"
+    x = torch.randn(2, 2048, hidden, generator=g)
+    up = lt.GeneralizedLinear(lt.GeneralizedMatrix(hidden, 2 * inter, layout, rank))
+    down = lt.GeneralizedLinear(lt.GeneralizedMatrix(inter, hidden, layout, rank))
+    assert tuple(up.weight.shape) == (4096, 56, 64) and tuple(down.weight.shape) == (16384, 7, 64)
+    with torch.no_grad():
+        for t in (up.weight, down.weight, up.matrix.lowrank_first, up.matrix.lowrank_second, down.matrix.lowrank_first,
+                  down.matrix.lowrank_second):
+            t.copy_(torch.randn(t.shape, generator=g) * 0.02)
+    dy = torch.randn(2, 2048, hidden, generator=g)
+    ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5, i2h_proj=up, h2o_proj=down).to(DEV).to(torch.bfloat16)
+    xd = x.to(DEV).requires_grad_(True)
+    y = ffn(xd)
+    names, params = zip(*ffn.named_parameters())
+    grads = torch.autograd.grad(y, [xd, *params], dy.to(DEV))
+    # oracle in fp32 on the GPU: dense expansion of the bf16-rounded sparse weights
+    leaves = {n: t.detach().float().clone().requires_grad_(True) for n, t in ffn.named_parameters()}
+
+    def proj(prefix, module):
+        return offn.LinearParams(leaves[f"{prefix}.matrix.weight"], leaves[f"{prefix}.bias"],
+                                 leaves[f"{prefix}.matrix.lowrank_first"], leaves[f"{prefix}.matrix.lowrank_second"],
+                                 module.matrix.forward_indices.cpu(), module.matrix.backward_indices.cpu(),
+                                 out_features=module.out_features)
+
+    def dense_on_device(lin):  # the oracle's dense expansion, vectorised (one scatter instead of 3584 concatenations)
+        in_f, A, b = lin.weight.shape
+        n_in, n_out = in_f // b, lin.out_features // b
+        w4 = lin.weight.reshape(n_in, A, b, b)
+        dense = torch.zeros(n_out, n_in, b, b, device=lin.weight.device)
+        ib = torch.arange(n_in, device=dense.device)[:, None].expand(n_in, A)
+        dense = dense.index_put((lin.backward_indices.to(dense.device), ib), w4)
+        return dense.permute(0, 2, 1, 3).reshape(n_out * b, in_f)
+
+    p = offn.FFNParams(leaves["pre_layer_norm.weight"], leaves["pre_layer_norm.bias"], proj("i2h_proj", ffn.i2h_proj),
+                       proj("h2o_proj", ffn.h2o_proj), cfg=offn.FFNConfig(gated=True, ln_eps=1e-5))
+    p.i2h.dense_weight = lambda lin=p.i2h: dense_on_device(lin)
+    p.h2o.dense_weight = lambda lin=p.h2o: dense_on_device(lin)
+    # the vectorised expansion is the oracle's block-by-block one (checked on the small down-projection's first rows)
+    small = offn.LinearParams(p.h2o.weight[:1024].detach().cpu(), backward_indices=p.h2o.backward_indices[:16],
+                              out_features=hidden)
+    assert torch.equal(small.dense_weight()[:, :1024], dense_on_device(p.h2o)[:, :1024].detach().cpu())
+    xr = x.to(DEV).requires_grad_(True)
+    y_ref = offn.plain_ffn(xr, p)
+    ref = torch.autograd.grad(y_ref, [xr, *[leaves[n] for n in names]], dy.to(DEV))
+    assert_close(y, y_ref.detach(), torch.bfloat16, "y")
+    assert_close(grads[0], ref[0], torch.bfloat16, "dx")
+    for name, a, b in zip(names, grads[1:], ref[1:]):
+        assert_close(a, b, torch.bfloat16, name)
+
+
 def test_saved_activation_memory_matches_reference_keep_set():
     """what stays alive between forward and backward is x (caller-owned), the pre-activation and 8 bytes of LayerNorm
     statistics per token -- the reference's keep-set (ffn.py:210-216)"""
