@@ -118,7 +118,7 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
   p.sp.mode = SPARSE_FWD; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
   p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
   p.sp.backward_indices = lin.backward_indices; p.sp.act = x; p.sp.ld_act = in; p.sp.weight = lin.weight;
-  return lt_launch_gemm_generic(p, kind, dtype, io_dtype, stream);
+  return lt_launch_gemm_sparse(p, kind, dtype, io_dtype, stream);
 }
 
 struct LinearBwdScratch {
@@ -168,7 +168,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.mode = SPARSE_DX; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
       p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.weight = lin.weight;
-      LT_TRY(lt_launch_gemm_generic(p, kind_dx, dtype, io_dtype, stream));
+      LT_TRY(lt_launch_gemm_sparse(p, kind_dx, dtype, io_dtype, stream));
     }
   }
   if (grads.bias) LT_TRY(lt_colsum(T, (int)out, out, dtype, dy, grads.bias, s.colsum, s.colsum_bytes, stream));
@@ -187,7 +187,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.act2 = x_act;
       p.sp.ld_act2 = in; p.sp.tokens = T;
       p.epi = epi_store_params(grads.weight, lin.block, dtype, nullptr);
-      LT_TRY(lt_launch_gemm_generic(p, EPI_STORE, dtype, io_dtype, stream));
+      LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));
     }
   }
   if (r > 0 && grads.lowrank_second) {  // dL2[out, r] = dy^T hid

@@ -29,6 +29,13 @@ typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int 
 
 __device__ __forceinline__ int swz_km(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int swz_mn(int k) { return ((k & 3) << 2) | (((k >> 3) & 1) << 1); }
+// mn-major tiles of COLS columns: the swizzle must stay inside a row's COLS / 8 chunks.  With 64 columns (128-byte rows,
+// two rows per 256-byte bank line) k-rows 2 apart and 8 apart are the ones that would collide in a transposing read.
+template <int COLS> __device__ __forceinline__ int swz_mn_cols(int k) {
+  static_assert(COLS == 64 || COLS % 128 == 0, "mn-major tile width");
+  if constexpr (COLS == 64) return (((k >> 1) & 1) << 1) | (((k >> 3) & 1) << 2);
+  else return swz_mn(k);
+}
 
 // scheduling hint for one k-substep: spread READS LDS-read instructions evenly between MFMAS matrix instructions
 template <int READS, int MFMAS, int G = 0> struct SchedInterleave {
@@ -40,9 +47,18 @@ template <int READS, int MFMAS, int G = 0> struct SchedInterleave {
   }
 };
 
-template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX>
+// SP != SPARSE_NONE: block-sparse walk with 64 x 64 blocks (see SparseWalk).  Each 64-wide k-step is one active block; its
+// operand tiles are fetched through the index tables, so nothing is gathered or scattered in HBM.  tiles_n then counts
+// groups: output blocks (FWD, tile 256 x 64), input blocks (DX, tile 256 x 64), or (input block, four of its active
+// output blocks) (DW, tile 256 x 64: four gathered dY column blocks against one X column block, reduced over tokens;
+// the four weight-gradient blocks are adjacent in the native [in_blocks, A, 64, 64] order).
+template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX, int SP = SPARSE_NONE>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int NT = WM * WN * 64;
+  static_assert(SP == SPARSE_NONE || (SP == SPARSE_FWD && A_KM && B_KM && BN == 64) ||
+                    (SP == SPARSE_DX && A_KM && !B_KM && BN == 64) ||
+                    (SP == SPARSE_DW && !A_KM && !B_KM && BM == 256 && BN == 64 && WM == 4 && WN == 1),
+                "operand layouts and tile shape of the block-sparse walks");
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int FM = WTM / 32, FN = WTN / 32;
   constexpr int A_CHUNKS = BM * BK / 8 / NT, B_CHUNKS = BN * BK / 8 / NT;  // 16-byte chunks per thread per stage
@@ -71,7 +87,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
   const int tm = first_m + (pid % group) % gsz;
   const int tn = (pid % group) / gsz;
   const int64_t m0 = (int64_t)tm * BM;
-  const int64_t n0 = (int64_t)tn * (gated ? BN / 2 : BN);  // gated: in gate columns
+  const int64_t n0 = (int64_t)tn * (gated ? BN / 2 : BN);  // gated: in gate columns; sparse FWD / DX: tn = block index
 
   f32x16 acc[FM][FN];
 #pragma unroll
@@ -83,17 +99,56 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
 
   u32x4 ra[A_CHUNKS], rb[B_CHUNKS];
 
-  const int kt_seg0 = (int)((p.K[0] + BK - 1) / BK);
-  const int kt_total = kt_seg0 + (p.nseg > 1 ? (int)((p.K[1] + BK - 1) / BK) : 0);
+  // k-steps: dense: segment 0 then segment 1; sparse FWD / DX: the active blocks of this group, then the low-rank segment
+  const SparseWalk& sp = p.sp;
+  const int sp_steps = SP == SPARSE_FWD ? sp.blocks_per_out : sp.blocks_per_in;
+  const int kt_seg0 = SP == SPARSE_NONE ? (int)((p.K[0] + BK - 1) / BK)
+                      : SP == SPARSE_DW ? (int)((sp.tokens + BK - 1) / BK)
+                                        : sp_steps;
+  const int kt_total = kt_seg0 + ((SP != SPARSE_DW && p.nseg > 1) ? (int)((p.K[1] + BK - 1) / BK) : 0);
+  // sparse DW: group tn = (input block, quad of its active output blocks a0 .. a0 + 3); a short last quad repeats the last
+  // block (computed, not stored)
+  int dw_ib = 0, dw_a0 = 0, dw_valid = 0;
+  int64_t dw_ob[4] = {0, 0, 0, 0};
+  if constexpr (SP == SPARSE_DW) {
+    const int quads = (sp.blocks_per_in + 3) / 4;
+    dw_ib = tn / quads;
+    dw_a0 = (tn % quads) * 4;
+    dw_valid = min(4, sp.blocks_per_in - dw_a0);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      dw_ob[j] = sp.backward_indices[(int64_t)dw_ib * sp.blocks_per_in + min(dw_a0 + j, sp.blocks_per_in - 1)];
+  }
 
   // global -> registers for k-step kt
   auto load_tiles = [&](int kt) {
     const int seg = kt >= kt_seg0;
-    const int64_t k0 = (int64_t)(seg ? kt - kt_seg0 : kt) * BK;
-    const int64_t K = p.K[seg];
+    int64_t k0 = (int64_t)(seg ? kt - kt_seg0 : kt) * BK;
+    int64_t K = p.K[seg];
     const bf16* A = reinterpret_cast<const bf16*>(p.A[seg].ptr);
     const bf16* B = reinterpret_cast<const bf16*>(p.B[seg].ptr);
-    const int64_t lda = p.A[seg].ld, ldb = p.B[seg].ld;
+    int64_t lda = p.A[seg].ld, ldb = p.B[seg].ld;
+    int64_t b_row0 = n0;  // first B row (k-major) / column (mn-major) of this tile
+    if constexpr (SP == SPARSE_FWD) {
+      if (!seg) {  // A: column block ib of X; B: weight block f, a [64 rows][64 k] matrix of its own
+        const int f = sp.forward_indices[(int64_t)tn * sp.blocks_per_out + kt];
+        A = reinterpret_cast<const bf16*>(sp.act); lda = sp.ld_act; k0 = (int64_t)(f / sp.blocks_per_in) * 64;
+        B = reinterpret_cast<const bf16*>(sp.weight) + (int64_t)f * 4096; ldb = 64; b_row0 = 0;
+        K = k0 + 64;
+      }
+    } else if constexpr (SP == SPARSE_DX) {
+      if (!seg) {  // A: column block ob of dY; B: weight block (ib, a) read as [64 k = output row][64 n = input column]
+        const int64_t ob = sp.backward_indices[(int64_t)tn * sp.blocks_per_in + kt];
+        A = reinterpret_cast<const bf16*>(sp.act); lda = sp.ld_act; k0 = ob * 64;
+        B = reinterpret_cast<const bf16*>(sp.weight) + ((int64_t)tn * sp.blocks_per_in + kt) * 4096 - k0 * 64; ldb = 64;
+        b_row0 = 0;
+        K = k0 + 64;
+      }
+    } else if constexpr (SP == SPARSE_DW) {  // A: four gathered dY column blocks; B: X column block ib; k = tokens
+      A = reinterpret_cast<const bf16*>(sp.act); lda = sp.ld_act;
+      B = reinterpret_cast<const bf16*>(sp.act2) + (int64_t)dw_ib * 64; ldb = sp.ld_act2; b_row0 = 0;
+      K = sp.tokens;
+    }
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; i++) {
       const int q = tid + i * NT;
@@ -104,7 +159,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       } else {
         const int kr = q / (BM / 8), c = q % (BM / 8);
         const int64_t gk = k0 + kr;
-        ra[i] = gk < K ? *reinterpret_cast<const u32x4*>(A + gk * lda + m0 + c * 8) : u32x4{0u, 0u, 0u, 0u};
+        int64_t col = m0 + c * 8;
+        if constexpr (SP == SPARSE_DW) col = dw_ob[c >> 3] * 64 + (c & 7) * 8;
+        ra[i] = gk < K ? *reinterpret_cast<const u32x4*>(A + gk * lda + col) : u32x4{0u, 0u, 0u, 0u};
       }
     }
 #pragma unroll
@@ -117,13 +174,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
           const int rr = row % WTN;
           gn = (rr / (WTN / 2)) * p.N + n0 + (row / WTN) * (WTN / 2) + rr % (WTN / 2);
         } else {
-          gn = n0 + row;
+          gn = b_row0 + row;
         }
-        rb[i] = *reinterpret_cast<const u32x4*>(B + gn * ldb + k0 + c * 8);
+        // a sparse FWD weight block holds its own 64 k: its columns start at 0, not at the gathered k0
+        const int64_t bk0 = (SP == SPARSE_FWD && !seg) ? 0 : k0;
+        rb[i] = *reinterpret_cast<const u32x4*>(B + gn * ldb + bk0 + c * 8);
       } else {
         const int kr = q / (BN / 8), c = q % (BN / 8);
         const int64_t gk = k0 + kr;
-        rb[i] = gk < K ? *reinterpret_cast<const u32x4*>(B + gk * ldb + n0 + c * 8) : u32x4{0u, 0u, 0u, 0u};
+        rb[i] = gk < K ? *reinterpret_cast<const u32x4*>(B + gk * ldb + b_row0 + c * 8) : u32x4{0u, 0u, 0u, 0u};
       }
     }
   };
@@ -137,7 +196,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
         *reinterpret_cast<u32x4*>(&lds_a[s][(row * 8 + (c ^ swz_km(row))) * 8]) = ra[i];
       } else {
         const int kr = q / (BM / 8), c = q % (BM / 8);
-        *reinterpret_cast<u32x4*>(&lds_a[s][kr * BM + ((c ^ swz_mn(kr)) << 3)]) = ra[i];
+        *reinterpret_cast<u32x4*>(&lds_a[s][kr * BM + ((c ^ swz_mn_cols<BM>(kr)) << 3)]) = ra[i];
       }
     }
 #pragma unroll
@@ -148,7 +207,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
         *reinterpret_cast<u32x4*>(&lds_b[s][(row * 8 + (c ^ swz_km(row))) * 8]) = rb[i];
       } else {
         const int kr = q / (BN / 8), c = q % (BN / 8);
-        *reinterpret_cast<u32x4*>(&lds_b[s][kr * BN + ((c ^ swz_mn(kr)) << 3)]) = rb[i];
+        *reinterpret_cast<u32x4*>(&lds_b[s][kr * BN + ((c ^ swz_mn_cols<BN>(kr)) << 3)]) = rb[i];
       }
     }
   };
@@ -158,14 +217,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     const int c = kk * 2 + (lane >> 5);
     return *reinterpret_cast<const bf16x8*>(&tile[(row * 8 + (c ^ swz_km(row))) * 8]);
   };
-  auto frag_mn = [&](const bf16* tile, int cols, int base, int kk) -> bf16x8 {
+  auto frag_mn = [&](const bf16* tile, auto cols_c, int base, int kk) -> bf16x8 {
+    constexpr int cols = decltype(cols_c)::value;
     union { bf16x8 v; s16x4 h[2]; } u;
     const int i16 = lane & 15;
     const int col = base + ((lane >> 4) & 1) * 16 + 4 * (i16 & 3);
 #pragma unroll
     for (int s = 0; s < 2; s++) {
       const int kr = kk * 16 + 8 * (lane >> 5) + 4 * s + (i16 >> 2);
-      const bf16* src = &tile[kr * cols + ((((col >> 3) ^ swz_mn(kr)) << 3) | (col & 7))];
+      const bf16* src = &tile[kr * cols + ((((col >> 3) ^ swz_mn_cols<cols>(kr)) << 3) | (col & 7))];
       u.h[s] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(src));
     }
     return u.v;
@@ -175,12 +235,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
 #pragma unroll
     for (int i = 0; i < FM; i++) {
       if constexpr (A_KM) a[i] = frag_km(lds_a[s], wm * WTM + i * 32, kk);
-      else a[i] = frag_mn(lds_a[s], BM, wm * WTM + i * 32, kk);
+      else a[i] = frag_mn(lds_a[s], std::integral_constant<int, BM>{}, wm * WTM + i * 32, kk);
     }
 #pragma unroll
     for (int j = 0; j < FN; j++) {
       if constexpr (B_KM) b[j] = frag_km(lds_b[s], wn * WTN + j * 32, kk);
-      else b[j] = frag_mn(lds_b[s], BN, wn * WTN + j * 32, kk);
+      else b[j] = frag_mn(lds_b[s], std::integral_constant<int, BN>{}, wn * WTN + j * 32, kk);
     }
   };
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);  // LDS read instructions per k-substep
@@ -216,6 +276,17 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
   //      writes HBM in 16-byte pieces of contiguous rows.  (The main loop ended with a barrier: the stages are free.)
   float* stage = reinterpret_cast<float*>(smem) + wave * (32 * STAGE_LD);
   const bool pair = (KIND == EPI_ACT_FWD) && gated;
+  // sparse DW: the tile is the [4 x 64][64] stack of weight-gradient blocks (ib, a0 .. a0 + 3), adjacent in memory
+  EpiParams epi = p.epi;
+  int64_t m_limit = p.M, n_base = n0 + wn * WTN, m_base = m0;
+  if constexpr (SP == SPARSE_DW) {
+    epi.out = reinterpret_cast<char*>(epi.out) +
+              ((int64_t)dw_ib * sp.blocks_per_in + dw_a0) * 4096 * (epi.out_dtype == LT_F32 ? 4 : 2);
+    epi.ldo = 64;
+    m_limit = dw_valid * 64;
+    n_base = 0;
+    m_base = 0;
+  }
 #pragma unroll
   for (int i = 0; i < FM; i++) {
 #pragma unroll
@@ -224,7 +295,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       for (int r = 0; r < 16; r++)
         stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * STAGE_LD + j * 32 + (lane & 31)] = acc[i][j][r];
     __builtin_amdgcn_wave_barrier();
-    const int64_t mrow0 = m0 + wm * WTM + i * 32;
+    const int64_t mrow0 = m_base + wm * WTM + i * 32;
     if (pair) {
       // columns [0, WTN/2) of the sub-tile are gate columns, [WTN/2, WTN) the matching linear columns
       constexpr int LANES_PER_ROW = WTN / 2 / 8, ROWS_PER_IT = 64 / LANES_PER_ROW;
@@ -244,15 +315,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
         const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW, c = (lane % LANES_PER_ROW) * 8;
         const int64_t m = mrow0 + row;
-        const int64_t n = n0 + wn * WTN + c;
+        const int64_t n = n_base + c;
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) v[e] = stage[row * STAGE_LD + c + e];
-        if (m < p.M) {
-          if constexpr (KIND == EPI_STORE) epi_store8(p.epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(p.epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8(p.epi, m, n, v);
-          else epi_out8<TX>(p.epi, m, n, v);
+        if (m < m_limit) {
+          if constexpr (KIND == EPI_STORE) epi_store8(epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8(epi, m, n, v);
+          else epi_out8<TX>(epi, m, n, v);
         }
       }
     }
@@ -686,6 +757,33 @@ int launch_cfg(const GemmProblem& p, int io_dtype, hipStream_t stream) {
   return LT_OK;
 }
 
+template <int KIND> int launch_sparse(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+  const SparseWalk& sp = p.sp;
+  const bool bf16_io = KIND == EPI_OUT && io_dtype == LT_BF16;
+  dim3 block(256);
+  if (sp.mode == SPARSE_FWD || sp.mode == SPARSE_DX) {
+    const int tiles_m = (int)((p.M + 255) / 256), groups = (int)(p.N / 64);
+    dim3 grid((unsigned)(tiles_m * groups));
+    if (sp.mode == SPARSE_FWD) {
+      if (bf16_io) hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, true, KIND, bf16, SPARSE_FWD>), grid, block, 0, stream, p, tiles_m, groups);
+      else hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, true, KIND, float, SPARSE_FWD>), grid, block, 0, stream, p, tiles_m, groups);
+    } else {
+      if (bf16_io) hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, false, KIND, bf16, SPARSE_DX>), grid, block, 0, stream, p, tiles_m, groups);
+      else hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, false, KIND, float, SPARSE_DX>), grid, block, 0, stream, p, tiles_m, groups);
+    }
+  } else {
+    if constexpr (KIND == EPI_STORE) {
+      const int groups = (int)((p.N / 64) * ((sp.blocks_per_in + 3) / 4));  // p.N = in_features
+      hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, false, false, EPI_STORE, float, SPARSE_DW>), dim3((unsigned)groups),
+                         block, 0, stream, p, 1, groups);
+    } else {
+      LT_FAIL(LT_ERR_UNSUPPORTED, "block-sparse weight gradient takes the plain store epilogue only");
+    }
+  }
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
 // the copy-based kernel addresses its operands with 32-bit byte offsets from a per-tile base
 bool dma_offsets_fit(const GemmProblem& p, int kind) {
   const bool gated = kind == EPI_ACT_FWD && p.epi.gated;
@@ -778,6 +876,50 @@ int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_
 }
 
 void lt_gemm_set_mfma_variant(int v) { g_mfma_variant = v; }
+
+// block-sparse walk on the matrix cores: 64 x 64 blocks, bf16, 16-byte aligned operands
+bool lt_sparse_mfma_supported(const GemmProblem& p, int kind) {
+  const SparseWalk& sp = p.sp;
+  const EpiParams& e = p.epi;
+  if (sp.mode == SPARSE_NONE || sp.block != 64 || p.M <= 0) return false;
+  if (kind == EPI_ACT_FWD && e.gated) return false;
+  if (sp.ld_act % 8 != 0 || !lt_aligned(sp.act, 16)) return false;
+  if (sp.mode == SPARSE_DW) {
+    if (kind != EPI_STORE || sp.ld_act2 % 8 != 0 || !lt_aligned(sp.act2, 16) || !lt_aligned(e.out, 16)) return false;
+    return true;
+  }
+  if (!lt_aligned(sp.weight, 16)) return false;
+  if (p.nseg > 1) {
+    if (p.K[1] <= 0 || p.K[1] % BK != 0 || p.A[1].ld % 8 != 0 || p.B[1].ld % 8 != 0 || !lt_aligned(p.A[1].ptr, 16) ||
+        !lt_aligned(p.B[1].ptr, 16))
+      return false;
+  }
+  if (e.bias && !lt_aligned(e.bias, 16)) return false;
+  if (kind == EPI_STORE && (e.ldo % 8 != 0 || !lt_aligned(e.out, 16))) return false;
+  if ((kind == EPI_ACT_FWD || kind == EPI_ACT_BWD) &&
+      (e.ld_pre % 8 != 0 || e.ld_hid % 8 != 0 || e.inter % 8 != 0 || !lt_aligned(e.pre, 16) ||
+       (e.hid && !lt_aligned(e.hid, 16)) || (e.dpre && !lt_aligned(e.dpre, 16))))
+    return false;
+  if (kind == EPI_OUT && (e.ldy % 8 != 0 || !lt_aligned(e.y, 16) || (e.x && !lt_aligned(e.x, 16)))) return false;
+  return true;
+}
+
+int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream) {
+  if (dtype != LT_BF16 || !lt_sparse_mfma_supported(p, kind)) return lt_launch_gemm_generic(p, kind, dtype, io_dtype, stream);
+  const SparseWalk& sp = p.sp;
+  const double steps = sp.mode == SPARSE_FWD ? sp.blocks_per_out : sp.blocks_per_in;
+  double flops = 2.0 * (double)p.M * (double)p.N * (steps * 64.0 + (p.nseg > 1 ? (double)p.K[1] : 0.0));
+  if (sp.mode == SPARSE_DW) flops = 2.0 * (double)sp.tokens * (double)(p.N / 64) * sp.blocks_per_in * 4096.0;
+  static const char* tags[4] = {"", "blocksparse_fwd_bf16", "blocksparse_dx_bf16", "blocksparse_dw_bf16"};
+  LtProfileScope scope(tags[sp.mode], flops, 0.0, stream);
+  switch (kind) {
+    case EPI_STORE: return launch_sparse<EPI_STORE>(p, io_dtype, stream);
+    case EPI_ACT_FWD: return launch_sparse<EPI_ACT_FWD>(p, io_dtype, stream);
+    case EPI_ACT_BWD: return launch_sparse<EPI_ACT_BWD>(p, io_dtype, stream);
+    case EPI_OUT: return launch_sparse<EPI_OUT>(p, io_dtype, stream);
+  }
+  LT_FAIL(LT_ERR_BAD_ARG, "unknown epilogue kind %d", kind);
+}
 
 int lt_launch_gemm(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream) {
   if (dtype == LT_BF16 && lt_gemm_mfma_supported(p, kind)) return lt_launch_gemm_mfma(p, kind, io_dtype, stream);

@@ -330,6 +330,8 @@ bool lt_gemm_mfma_supported(const GemmProblem& p, int kind);
 int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_t stream);
 // algorithmic flops of a dense problem: 2 * M * N * (K0 + K1)
 double lt_gemm_flops(const GemmProblem& p, int kind);
+// block-sparse walk: matrix-core kernel for 64 x 64 bf16 blocks, else the any-shape kernel
+int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);
 // 0: choose; 1: register-staged tiled kernel; 2: copy-based tiled kernel
 void lt_gemm_set_mfma_variant(int v);
 // picks the tiled kernel when it applies and dtype is bf16, else the any-shape kernel
