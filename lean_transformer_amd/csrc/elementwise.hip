@@ -388,6 +388,26 @@ __global__ void dropout_mask_kernel(int64_t n, uint8_t* __restrict__ keep, Dropo
   keep[idx] = drop.p > 0.f ? (dropout_keep(drop, idx) ? 1 : 0) : 1;
 }
 
+// sum of split-k partial results in slice order, 4 elements per thread
+template <typename TO>
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t stride, int64_t count, int cols,
+                                     const float* __restrict__ bias, TO* __restrict__ out) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= count) return;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < slices; s++) {
+    float v[4];
+    load4(partial + (int64_t)s * stride + i, v);
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[e] += v[e];
+  }
+  if (bias) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[e] += bias[(i + e) % cols];
+  }
+  store4(out + i, acc);
+}
+
 inline unsigned blocks_for(int64_t n, int threads) { return (unsigned)((n + threads - 1) / threads); }
 
 }  // namespace
@@ -609,6 +629,20 @@ int lt_dropout_cast(int64_t n, int in_dtype, const void* in, int out_dtype, void
 int lt_dropout_mask_launch(int64_t n, uint8_t* keep, const DropoutParams& drop, hipStream_t stream) {
   LT_REQUIRE(n > 0 && keep, LT_ERR_BAD_ARG, "dropout mask: bad arguments");
   hipLaunchKernelGGL(dropout_mask_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, n, keep, drop);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t count, int cols, const float* bias,
+                     int out_dtype, void* out, hipStream_t stream) {
+  LT_REQUIRE(partial && out && slices > 0 && count > 0 && (count & 3) == 0 && (stride & 3) == 0, LT_ERR_BAD_ARG,
+             "split-k reduce: bad arguments");
+  LtProfileScope scope("splitk_reduce", 0.0, (double)count * (4.0 * slices + lt_dtype_size(out_dtype)), stream);
+  dim3 grid(blocks_for(count / 4, 256)), block(256);
+  if (out_dtype == LT_F32)
+    hipLaunchKernelGGL((splitk_reduce_kernel<float>), grid, block, 0, stream, partial, slices, stride, count, cols, bias, (float*)out);
+  else
+    hipLaunchKernelGGL((splitk_reduce_kernel<bf16>), grid, block, 0, stream, partial, slices, stride, count, cols, bias, (bf16*)out);
   LT_LAUNCH_CHECK();
   return LT_OK;
 }

@@ -87,7 +87,8 @@ GemmProblem blank_problem() {
 // y-side of one generalized linear layer: [lowrank_hid = x L1^T], then x W^T (+ lowrank_hid L2^T) through epilogue `kind`.
 // For a gated EPI_ACT_FWD the epilogue pairs output column n with n + out_features / 2.
 int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* x, int kind, const EpiParams& epi,
-                        void* lowrank_hid, int io_dtype, hipStream_t stream) {
+                        void* lowrank_hid, int io_dtype, hipStream_t stream, void* skinny_ws = nullptr,
+                        size_t skinny_bytes = 0) {
   const int64_t in = lin.in_features, out = lin.out_features, r = lin.lowrank;
   if (r > 0) {
     LT_REQUIRE(lowrank_hid, LT_ERR_BAD_ARG, "linear forward: lowrank_hid buffer missing");
@@ -96,7 +97,7 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
     q.A[0] = operand(x, in, true);
     q.B[0] = operand(lin.lowrank_first, in, true);
     q.epi = epi_store_params(lowrank_hid, r, dtype, nullptr);
-    LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+    LT_TRY(lt_launch_gemm_skinny(q, dtype, io_dtype, skinny_ws, skinny_bytes, stream));
   }
   GemmProblem p = blank_problem();
   const bool gated = kind == EPI_ACT_FWD && epi.gated;
@@ -125,12 +126,16 @@ struct LinearBwdScratch {
   void* g_hid;     // [T, r] dtype
   void* colsum;    // lt_colsum_workspace(T, out)
   size_t colsum_bytes;
+  void* skinny;    // split-k partial sums of the low-rank GEMMs
+  size_t skinny_bytes;
 };
 
 void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, LinearBwdScratch& s) {
   s.g_hid = lin.lowrank > 0 ? ws.take((size_t)T * lin.lowrank * lt_dtype_size(dtype)) : nullptr;
   s.colsum_bytes = lt_colsum_workspace(T, lin.out_features);
   s.colsum = ws.take(s.colsum_bytes);
+  s.skinny_bytes = lin.lowrank > 0 ? lt_gemm_skinny_workspace(T, lin.lowrank) : 0;
+  s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 
 // gradient side of one generalized linear layer.  The input-gradient GEMM runs FIRST, through epilogue `kind_dx`
@@ -147,7 +152,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
     q.A[0] = operand(dy, out, true);
     q.B[0] = operand(lin.lowrank_second, r, false);
     q.epi = epi_store_params(s.g_hid, r, dtype, nullptr);
-    LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+    LT_TRY(lt_launch_gemm_skinny(q, dtype, io_dtype, s.skinny, s.skinny_bytes, stream));
   }
   if (need_dx) {  // dx = dy W (+ g_hid L1)
     GemmProblem p = blank_problem();
@@ -197,7 +202,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
     q.A[0] = operand(dy, out, false);
     q.B[0] = operand(lowrank_hid, r, false);
     q.epi = epi_store_params(grads.lowrank_second, r, dtype, nullptr);
-    LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+    LT_TRY(lt_launch_gemm_skinny(q, dtype, io_dtype, s.skinny, s.skinny_bytes, stream));
   }
   if (r > 0 && grads.lowrank_first) {  // dL1[r, in] = g_hid^T x
     GemmProblem q = blank_problem();
@@ -205,7 +210,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
     q.A[0] = operand(s.g_hid, r, false);
     q.B[0] = operand(x_act, in, false);
     q.epi = epi_store_params(grads.lowrank_first, in, dtype, nullptr);
-    LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+    LT_TRY(lt_launch_gemm_skinny(q, dtype, io_dtype, s.skinny, s.skinny_bytes, stream));
   }
   return LT_OK;
 }
@@ -231,14 +236,19 @@ int check_ffn_desc(const lt_ffn_desc* d) {
 }
 
 struct FwdScratch {
-  void* u;    // [T, H] compute dtype: LayerNorm output
-  void* hid;  // [T, I] compute dtype: activation output
+  void* u;       // [T, H] compute dtype: LayerNorm output
+  void* hid;     // [T, I] compute dtype: activation output
+  void* skinny;  // split-k partial sums of the low-rank GEMMs
+  size_t skinny_bytes;
 };
 
 void plan_forward(const lt_ffn_desc& d, Bump& ws, FwdScratch& s) {
   const size_t e = lt_dtype_size(d.compute_dtype);
   s.u = ws.take((size_t)d.tokens * d.hidden * e);
   s.hid = ws.take((size_t)d.tokens * d.intermediate * e);
+  const int r = d.i2h.lowrank > d.h2o.lowrank ? d.i2h.lowrank : d.h2o.lowrank;
+  s.skinny_bytes = r > 0 ? lt_gemm_skinny_workspace(d.tokens, r) : 0;
+  s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 
 struct BwdScratch {
@@ -316,27 +326,27 @@ extern "C" int lt_ffn_forward(const lt_ffn_desc* desc, const void* x, void* y, c
   if (d.i2h.block > 0 && d.gated) {
     // the block-sparse walk has no paired-column epilogue: store P, then a separate activation pass
     EpiParams e = epi_store_params(saved->pre_activation, N1, cdt, d.i2h.bias);
-    LT_TRY(linear_forward_impl(d.i2h, T, cdt, s.u, EPI_STORE, e, saved->i2h_lowrank_hid, io, stream));
+    LT_TRY(linear_forward_impl(d.i2h, T, cdt, s.u, EPI_STORE, e, saved->i2h_lowrank_hid, io, stream, s.skinny, s.skinny_bytes));
     LT_TRY(lt_act_forward(T, I, 1, d.act, cdt, saved->pre_activation, s.hid, stream));
   } else {
     EpiParams e;
     memset(&e, 0, sizeof(e));
     e.bias = d.i2h.bias; e.pre = saved->pre_activation; e.ld_pre = N1; e.hid = s.hid; e.ld_hid = I;
     e.gated = d.gated; e.act = d.act; e.inter = I;
-    LT_TRY(linear_forward_impl(d.i2h, T, cdt, s.u, EPI_ACT_FWD, e, saved->i2h_lowrank_hid, io, stream));
+    LT_TRY(linear_forward_impl(d.i2h, T, cdt, s.u, EPI_ACT_FWD, e, saved->i2h_lowrank_hid, io, stream, s.skinny, s.skinny_bytes));
   }
 
   // down-projection (+ post-LN) + dropout + residual
   if (d.post_ln_weight) {
     EpiParams e = epi_store_params(saved->post_ln_input, H, cdt, d.h2o.bias);
-    LT_TRY(linear_forward_impl(d.h2o, T, cdt, s.hid, EPI_STORE, e, saved->h2o_lowrank_hid, io, stream));
+    LT_TRY(linear_forward_impl(d.h2o, T, cdt, s.hid, EPI_STORE, e, saved->h2o_lowrank_hid, io, stream, s.skinny, s.skinny_bytes));
     LT_TRY(lt_ln_forward(T, (int)H, d.ln_eps, cdt, saved->post_ln_input, d.post_ln_weight, d.post_ln_bias, io, y, nullptr,
                          io, d.residual ? x : nullptr, &drop, true, stream));
   } else {
     EpiParams e;
     memset(&e, 0, sizeof(e));
     e.bias = d.h2o.bias; e.x = d.residual ? x : nullptr; e.y = y; e.ldy = H; e.drop = drop;
-    LT_TRY(linear_forward_impl(d.h2o, T, cdt, s.hid, EPI_OUT, e, saved->h2o_lowrank_hid, io, stream));
+    LT_TRY(linear_forward_impl(d.h2o, T, cdt, s.hid, EPI_OUT, e, saved->h2o_lowrank_hid, io, stream, s.skinny, s.skinny_bytes));
   }
   return LT_OK;
 }

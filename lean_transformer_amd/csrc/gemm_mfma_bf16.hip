@@ -17,6 +17,7 @@
 //
 // Workgroups are numbered so that each XCD (hardware dispatches workgroup i to XCD i % 8) walks a contiguous range of
 // tiles, GROUP_M tile-rows at a time, keeping one XCD's 32 concurrent tiles on few distinct A / B panels in its own L2.
+#include <algorithm>
 #include <type_traits>
 
 #include "lt_gemm.h"
@@ -245,12 +246,21 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
   };
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);  // LDS read instructions per k-substep
 
-  load_tiles(0);
-  store_tiles(0);
+  // split-k: this workgroup's slice of the k-steps
+  int kt_begin = 0, kt_end = kt_total;
+  if (p.ksplit > 1) {
+    const int per = (kt_total + p.ksplit - 1) / p.ksplit;
+    kt_begin = min(kt_total, (int)blockIdx.y * per);
+    kt_end = min(kt_total, kt_begin + per);
+  }
+  if (kt_begin < kt_end) {
+    load_tiles(kt_begin);
+    store_tiles(kt_begin & 1);
+  }
   __syncthreads();
-  for (int kt = 0; kt < kt_total; kt++) {
+  for (int kt = kt_begin; kt < kt_end; kt++) {
     const int s = kt & 1;
-    const bool has_next = kt + 1 < kt_total;
+    const bool has_next = kt + 1 < kt_end;
     if (has_next) load_tiles(kt + 1);
     // fragments are double-buffered in registers: the LDS reads of k-substep kk + 1 are issued before, and interleaved
     // with, the MFMAs of k-substep kk
@@ -279,6 +289,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
   // sparse DW: the tile is the [4 x 64][64] stack of weight-gradient blocks (ib, a0 .. a0 + 3), adjacent in memory
   EpiParams epi = p.epi;
   int64_t m_limit = p.M, n_base = n0 + wn * WTN, m_base = m0;
+  if (p.ksplit > 1) epi.out = reinterpret_cast<float*>(epi.out) + (int64_t)blockIdx.y * p.split_stride;
   if constexpr (SP == SPARSE_DW) {
     epi.out = reinterpret_cast<char*>(epi.out) +
               ((int64_t)dw_ib * sp.blocks_per_in + dw_a0) * 4096 * (epi.out_dtype == LT_F32 ? 4 : 2);
@@ -876,6 +887,60 @@ int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_
 }
 
 void lt_gemm_set_mfma_variant(int v) { g_mfma_variant = v; }
+
+namespace {
+template <bool A_KM, bool B_KM> int launch_skinny(const GemmProblem& p, int slices, hipStream_t stream) {
+  const int tiles_m = (int)((p.M + 127) / 128), tiles_n = (int)(p.N / 128);
+  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)slices), block(256);
+  hipLaunchKernelGGL((gemm_bf16_kernel<128, 128, 2, 2, A_KM, B_KM, EPI_STORE, float>), grid, block, 0, stream, p, tiles_m, tiles_n);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+constexpr int SKINNY_MAX_SLICES = 16;
+}  // namespace
+
+// partial sums of up to SKINNY_MAX_SLICES slices of a [tokens, lowrank] (or equally large) fp32 result
+size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank) {
+  return lt_align_up((size_t)SKINNY_MAX_SLICES * (size_t)tokens * (size_t)lowrank * sizeof(float), 256);
+}
+
+int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
+                          hipStream_t stream) {
+  const bool a_km = p.A[0].kmajor, b_km = p.B[0].kmajor;
+  const EpiParams& e = p.epi;
+  bool ok = dtype == LT_BF16 && p.nseg == 1 && p.sp.mode == SPARSE_NONE && p.M > 0 && p.N > 0 && p.N % 128 == 0 &&
+            !(!a_km && b_km) && (a_km || p.M % 128 == 0) && ((!a_km && !b_km) || p.K[0] % BK == 0) && p.K[0] > 0 &&
+            p.A[0].ld % 8 == 0 && p.B[0].ld % 8 == 0 && lt_aligned(p.A[0].ptr, 16) && lt_aligned(p.B[0].ptr, 16) &&
+            e.ldo == p.N && lt_aligned(e.out, 16) && (!e.bias || lt_aligned(e.bias, 16));
+  // shapes the 256 x 256 kernels fill the chip with keep going there
+  const int64_t tiles = ((p.M + 127) / 128) * (p.N / 128);
+  if (ok && lt_gemm_mfma_supported(p, EPI_STORE) && ((p.M + 255) / 256) * (p.N / 256) >= 128) ok = false;
+  if (!ok) return lt_launch_gemm(p, EPI_STORE, dtype, io_dtype, stream);
+  const int kt_total = (int)((p.K[0] + BK - 1) / BK);
+  int slices = 1;
+  if (workspace && tiles < 192) {
+    slices = (int)std::min<int64_t>(std::min<int64_t>(256 / tiles, kt_total / 4), SKINNY_MAX_SLICES);
+    const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.M * (size_t)p.N * sizeof(float)));
+    slices = (int)std::max<int64_t>(1, std::min<int64_t>(slices, fit));
+  }
+  GemmProblem q = p;
+  if (slices > 1) {
+    q.ksplit = slices;
+    q.split_stride = p.M * p.N;
+    q.epi.out = workspace;
+    q.epi.out_dtype = LT_F32;
+    q.epi.bias = nullptr;
+  }
+  {
+    LtProfileScope scope("gemm_bf16_skinny", lt_gemm_flops(p, EPI_STORE), 0.0, stream);
+    int status;
+    if (a_km && b_km) status = launch_skinny<true, true>(q, slices, stream);
+    else if (a_km) status = launch_skinny<true, false>(q, slices, stream);
+    else status = launch_skinny<false, false>(q, slices, stream);
+    if (status != LT_OK || slices == 1) return status;
+  }
+  return lt_splitk_reduce((const float*)workspace, slices, p.M * p.N, p.M * p.N, (int)p.N, e.bias, e.out_dtype, e.out, stream);
+}
 
 // block-sparse walk on the matrix cores: 64 x 64 blocks, bf16, 16-byte aligned operands
 bool lt_sparse_mfma_supported(const GemmProblem& p, int kind) {

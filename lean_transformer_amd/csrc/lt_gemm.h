@@ -70,6 +70,10 @@ struct GemmProblem {
   GemmOperand A[2], B[2];
   EpiParams epi;
   SparseWalk sp;  // sp.mode == SPARSE_NONE for a dense problem
+  // split-k (tiled kernel, EPI_STORE only): blockIdx.y = slice of the k-steps; slice s stores fp32 partial sums at
+  // epi.out + s * split_stride elements, summed afterwards in slice order (deterministic)
+  int ksplit;
+  int64_t split_stride;
 };
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -332,6 +336,15 @@ int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_
 double lt_gemm_flops(const GemmProblem& p, int kind);
 // block-sparse walk: matrix-core kernel for 64 x 64 bf16 blocks, else the any-shape kernel
 int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);
+// EPI_STORE problems with few output tiles and a long reduction (the low-rank factors of a generalized linear layer):
+// 128 x 128 tiles, the reduction split over workgroups through `workspace` when that fills the chip better.  Falls back to
+// lt_launch_gemm when the shape does not fit.
+size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank);
+int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
+                          hipStream_t stream);
+// out[i] = sum_s partial[s * stride + i] (+ bias[i % cols]) for i < count, cast to out_dtype
+int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t count, int cols, const float* bias,
+                     int out_dtype, void* out, hipStream_t stream);
 // 0: choose; 1: register-staged tiled kernel; 2: copy-based tiled kernel
 void lt_gemm_set_mfma_variant(int v);
 // picks the tiled kernel when it applies and dtype is bf16, else the any-shape kernel
