@@ -18,6 +18,7 @@
 // Workgroups are numbered so that each XCD (hardware dispatches workgroup i to XCD i % 8) walks a contiguous range of
 // tiles, GROUP_M tile-rows at a time, keeping one XCD's 32 concurrent tiles on few distinct A / B panels in its own L2.
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "lt_gemm.h"
@@ -384,9 +385,15 @@ template <int READS, int COPIES, int MFMAS, int G = 0> struct SchedInterleave3 {
 // that older copies have landed; the empty asm statements only keep it from moving LDS accesses across the barrier.
 template <int N> __device__ __forceinline__ void wait_copies_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+#ifdef LT_DBG_NO_WAIT
+  __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));
+#else
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));  // vmcnt(N) expcnt(7: none) lgkmcnt(0)
+#endif
   asm volatile("" ::: "memory");
+#ifndef LT_DBG_NO_BARRIER
   __builtin_amdgcn_s_barrier();
+#endif
   asm volatile("" ::: "memory");
 }
 
@@ -430,6 +437,9 @@ template <bool KM> struct DmaOperand {
 
   // all copies of unit u (counted inside the k-segment) into `dst`; k_limit: reduction length for the ragged test
   template <bool K_TAIL> __device__ __forceinline__ void issue(int u, bf16* dst, int wave, int64_t k_limit) const {
+#ifdef LT_DBG_NO_COPY
+    return;
+#endif
 #pragma unroll
     for (int j = 0; j < LOADS; j++) {
       const char* g = base + u * unit_bytes + off[j];
@@ -500,6 +510,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     else return i == 0 ? b_s0 : i == 1 ? b_s1 : i == 2 ? b_s2 : b_s3;
   };
 
+  // Workgroups start their walk over k at different offsets and wrap around: with a power-of-two leading dimension every
+  // row of a k-major tile otherwise maps to the same memory channels at the same time, chip-wide.  The offset is the same
+  // for the workgroups of one XCD that run next to each other (they share operand panels through that XCD's L2) and
+  // differs between XCDs.  Measured on the up- and down-projection shapes: +16 % and +25 % for two k-major operands,
+  // nothing to gain for mn-major ones.
+  int rot = 0;
+  if (!K_TAIL && p.nseg == 1 && (kt_total & 1) == 0 && p.krot) {
+    const unsigned bx = blockIdx.x;
+    const unsigned r = (bx & 7) * (kt_total >> 3) +
+                       (p.krot == 1 ? ((bx >> 3) & 3) * (kt_total >> 5) : ((bx >> 3) & 7) * (kt_total >> 6));
+    rot = __builtin_amdgcn_readfirstlane((int)((r % (unsigned)kt_total) & ~1u));
+  }
+  auto rotated = [&](int ks) {
+    const int r = ks + rot;
+    return r >= kt_total ? r - kt_total : r;
+  };
   DmaOperand<A_KM> ca;
   DmaOperand<B_KM> cb;
   auto setup_a = [&](int seg) { ca.setup(p.A[seg], seg, m0, A_KM ? p.M : 0, 0, wave, lane); };
@@ -513,7 +539,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       seg = t >= kt_seg0;
       if (seg != ca.seg) setup_a(seg);
     }
-    const int ks = seg ? t - kt_seg0 : t;
+    const int ks = rotated(seg ? t - kt_seg0 : t);
     ca.template issue<K_TAIL>(A_KM ? ks >> 1 : ks, a_buf(I), wave, p.K[seg]);
   };
   auto copy_b = [&](auto steady, auto I, int t) {
@@ -522,7 +548,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       seg = t >= kt_seg0;
       if (seg != cb.seg) setup_b(seg);
     }
-    const int ks = seg ? t - kt_seg0 : t;
+    const int ks = rotated(seg ? t - kt_seg0 : t);
     cb.template issue<K_TAIL>(B_KM ? ks >> 1 : ks, b_buf(I), wave, p.K[seg]);
   };
 
@@ -728,7 +754,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 }
 
 template <bool A_KM, bool B_KM, int KIND>
-int launch_dma(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+int launch_dma(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
+  GemmProblem p = problem;
+  // k-walk stagger: on unless the caller chose (15: off)
+  if (p.krot == 0) p.krot = (A_KM && B_KM) ? 2 : 0;
+  else if (p.krot == 15) p.krot = 0;
   const bool gated = KIND == EPI_ACT_FWD && p.epi.gated;
   const int tiles_m = (int)((p.M + 255) / 256);
   const int tiles_n = (int)(p.N / (gated ? 128 : 256));

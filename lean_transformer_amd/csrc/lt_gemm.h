@@ -74,6 +74,7 @@ struct GemmProblem {
   // epi.out + s * split_stride elements, summed afterwards in slice order (deterministic)
   int ksplit;
   int64_t split_stride;
+  int krot;  // copy-based kernel: how workgroups stagger their walk over k (0: all start at k = 0)
 };
 
 // ---------------------------------------------------------------------------------------------------------------------
