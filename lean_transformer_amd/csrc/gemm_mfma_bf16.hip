@@ -452,6 +452,41 @@ template <bool KM> struct DmaOperand {
   }
 };
 
+// Copies complete in issue order, so the wait before the barrier of k-step t names how many of the youngest copies may
+// still be in flight: those issued after the last copy k-step t + 1 reads.  This replays the issue order of the steady
+// loop (first half of s: mn-major A and B for s + 3 [B only when not split], then on even s the k-major blocks of
+// s + 2 [A only when not late]; second half of s, after its barrier: split mn-major B for s + 3, on odd s the late
+// k-major A block of s + 3) and counts them.
+constexpr int copies_in_flight(bool a_km, bool b_km, bool a_late, bool b_split, int parity) {
+  const int t = 8 + parity;
+  int counts[64] = {}, needed[64] = {}, n = 0;
+  for (int s = t - 8; s <= t; s++) {
+    if (!a_km) { counts[n] = 4; needed[n++] = s + 3; }
+    if (!b_km && !b_split) { counts[n] = 4; needed[n++] = s + 3; }
+    if (a_km && !a_late && s % 2 == 0) { counts[n] = 8; needed[n++] = s + 2; }
+    if (b_km && s % 2 == 0) { counts[n] = 8; needed[n++] = s + 2; }
+    if (s == t) break;
+    if (!b_km && b_split) { counts[n] = 4; needed[n++] = s + 3; }
+    if (a_km && a_late && s % 2 == 1) { counts[n] = 8; needed[n++] = s + 3; }
+  }
+  int last = -1;
+  for (int i = 0; i < n; i++)
+    if (needed[i] <= t + 1) last = i;
+  int sum = 0;
+  for (int i = last + 1; i < n; i++) sum += counts[i];
+  return sum;
+}
+static_assert(copies_in_flight(false, false, false, false, 0) == 16 && copies_in_flight(true, true, false, false, 1) == 0 &&
+              copies_in_flight(true, true, false, false, 0) == 16 && copies_in_flight(true, false, false, false, 1) == 4 &&
+              copies_in_flight(true, false, false, false, 0) == 16, "issue-order model");
+
+#ifndef LT_A_LATE
+#define LT_A_LATE 1
+#endif
+#ifndef LT_B_SPLIT
+#define LT_B_SPLIT 1
+#endif
+
 template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
@@ -597,17 +632,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   //                   matrix instructions on the second 16 k
   // I = t mod 4 at compile time.  steady == true: straight-line code, valid while every copy it issues exists and stays
   // inside the current k-segment.
+  // Copies are spread over the half-steps so that the address unit, which the four wavefronts share, is not handed a
+  // whole block at once: a k-major A block goes out in the second half of odd k-steps (A_LATE), mn-major B in the second
+  // half of every k-step (B_SPLIT); the rest in the first half.
+  constexpr bool A_LATE = A_KM && LT_A_LATE, B_SPLIT = !B_KM && !A_KM && LT_B_SPLIT;
   auto first_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
     load_frags(I, 1, af[1], bfr[1]);
     if (STEADY || t + 3 < kt_total) {  // mn-major: k-step t + 3 into the tile freed by the last barrier
       if constexpr (!A_KM) copy_a(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
-      if constexpr (!B_KM) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+      if constexpr (!B_KM && !B_SPLIT) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
     }
     if constexpr ((i & 1) == 0 && N_KM > 0) {  // k-major: the block of k-steps t + 2, t + 3 into the other buffer
       if (STEADY || t + 2 < kt_total) {
-        if constexpr (A_KM) copy_a(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
+        if constexpr (A_KM && !A_LATE) copy_a(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
         if constexpr (B_KM) copy_b(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
       }
     }
@@ -615,22 +654,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     for (int x = 0; x < FM; x++)
 #pragma unroll
       for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][x], bfr[0][y], acc[x][y], 0, 0, 0);
-    SchedInterleave3<FRAG_READS, N_MN + ((i & 1) == 0 ? N_KM : 0), FM * FN>::run();
+    constexpr int COPIES = (A_KM ? 0 : 4) + ((B_KM || B_SPLIT) ? 0 : 4) +
+                           ((i & 1) == 0 ? ((A_KM && !A_LATE) ? 8 : 0) + (B_KM ? 8 : 0) : 0);
+    SchedInterleave3<FRAG_READS, COPIES, FM * FN>::run();
   };
   auto second_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
-    // Copies complete in issue order.  Issued after the ones k-step t + 1 needs, and therefore allowed in flight:
-    //   t even: mn(t + 2), mn(t + 3), km(block of t + 2)      t odd: mn(t + 3) only (the block of t + 1 must have landed)
-    constexpr int IN_FLIGHT = N_KM == 0 ? 2 * N_MN : ((i & 1) == 0 ? 2 * N_MN + N_KM : N_MN);
+    constexpr int IN_FLIGHT = copies_in_flight(A_KM, B_KM, A_LATE, B_SPLIT, i & 1);
     if constexpr (STEADY) wait_copies_and_barrier<IN_FLIGHT>();
     else wait_copies_and_barrier<0>();
     if (STEADY || t + 1 < kt_total) load_frags(std::integral_constant<int, (i + 1) & 3>{}, 0, af[0], bfr[0]);
+    if (STEADY || t + 3 < kt_total) {
+      // the barrier above freed the buffers of k-step t - 1 and, on odd t, the k-major buffer of k-steps t - 1, t
+      if constexpr (B_SPLIT) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+      if constexpr (A_LATE && (i & 1) == 1) copy_a(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+    }
 #pragma unroll
     for (int x = 0; x < FM; x++)
 #pragma unroll
       for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][x], bfr[1][y], acc[x][y], 0, 0, 0);
-    SchedInterleave3<FRAG_READS, 0, FM * FN>::run();
+    constexpr int COPIES = (B_SPLIT ? 4 : 0) + ((A_LATE && (i & 1) == 1) ? 8 : 0);
+    SchedInterleave3<FRAG_READS, COPIES, FM * FN>::run();
   };
   using Steady = std::integral_constant<bool, true>;
   using Ragged = std::integral_constant<bool, false>;
@@ -651,6 +696,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   if (kt_total > 2) {
     if constexpr (!A_KM) copy_a(Ragged{}, P2{}, 2);
     if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2);
+    if constexpr (A_LATE) copy_a(Ragged{}, P2{}, 2);  // the second block; later ones follow from the odd k-steps
   }
   wait_copies_and_barrier<0>();
   load_frags(P0{}, 0, af[0], bfr[0]);
