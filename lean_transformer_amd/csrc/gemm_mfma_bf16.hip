@@ -436,12 +436,11 @@ template <bool KM> struct DmaOperand {
   }
 
   // all copies of unit u (counted inside the k-segment) into `dst`; k_limit: reduction length for the ragged test
-  template <bool K_TAIL> __device__ __forceinline__ void issue(int u, bf16* dst, int wave, int64_t k_limit) const {
-#ifdef LT_DBG_NO_COPY
-    return;
-#endif
+  // J0, J1: range of this wavefront's copy instructions (a k-major block can go out in two halves)
+  template <bool K_TAIL, int J0 = 0, int J1 = LOADS>
+  __device__ __forceinline__ void issue(int u, bf16* dst, int wave, int64_t k_limit) const {
 #pragma unroll
-    for (int j = 0; j < LOADS; j++) {
+    for (int j = J0; j < J1; j++) {
       const char* g = base + u * unit_bytes + off[j];
       if constexpr (K_TAIL && !KM) {
         if ((int64_t)u * DK + krow[j] >= k_limit) g = reinterpret_cast<const char*>(&lt_zero_chunk);
@@ -452,22 +451,33 @@ template <bool KM> struct DmaOperand {
   }
 };
 
+// Where the two halves (4 copy instructions per wavefront each) of a k-major block go out.  The buffer of the block that
+// holds k-steps 2b + 2, 2b + 3 is free after the barrier of k-step 2b - 1 and must be full at the barrier of 2b + 1:
+//   slot 0: second half of k-step 2b - 1      slot 1: first half of 2b      slot 2: second half of 2b
+struct BlockSlots {
+  int half[2];
+};
+
 // Copies complete in issue order, so the wait before the barrier of k-step t names how many of the youngest copies may
 // still be in flight: those issued after the last copy k-step t + 1 reads.  This replays the issue order of the steady
-// loop (first half of s: mn-major A and B for s + 3 [B only when not split], then on even s the k-major blocks of
-// s + 2 [A only when not late]; second half of s, after its barrier: split mn-major B for s + 3, on odd s the late
-// k-major A block of s + 3) and counts them.
-constexpr int copies_in_flight(bool a_km, bool b_km, bool a_late, bool b_split, int parity) {
+// loop and counts them.  First half of s: mn-major A and B for s + 3 (B only when not split), then on even s the slot-1
+// halves of the k-major blocks of s + 2; second half of s, after its barrier: split mn-major B for s + 3, then on odd s
+// the slot-0 halves of the blocks of s + 3, on even s the slot-2 halves of the blocks of s + 2.
+constexpr int copies_in_flight(bool a_km, bool b_km, BlockSlots sa, BlockSlots sb, bool b_split, int parity) {
   const int t = 8 + parity;
-  int counts[64] = {}, needed[64] = {}, n = 0;
+  int counts[128] = {}, needed[128] = {}, n = 0;
   for (int s = t - 8; s <= t; s++) {
     if (!a_km) { counts[n] = 4; needed[n++] = s + 3; }
     if (!b_km && !b_split) { counts[n] = 4; needed[n++] = s + 3; }
-    if (a_km && !a_late && s % 2 == 0) { counts[n] = 8; needed[n++] = s + 2; }
-    if (b_km && s % 2 == 0) { counts[n] = 8; needed[n++] = s + 2; }
+    if (s % 2 == 0) {
+      for (int h = 0; h < 2; h++) if (a_km && sa.half[h] == 1) { counts[n] = 4; needed[n++] = s + 2; }
+      for (int h = 0; h < 2; h++) if (b_km && sb.half[h] == 1) { counts[n] = 4; needed[n++] = s + 2; }
+    }
     if (s == t) break;
     if (!b_km && b_split) { counts[n] = 4; needed[n++] = s + 3; }
-    if (a_km && a_late && s % 2 == 1) { counts[n] = 8; needed[n++] = s + 3; }
+    const int want = s % 2 ? 0 : 2, first = s % 2 ? s + 3 : s + 2;
+    for (int h = 0; h < 2; h++) if (a_km && sa.half[h] == want) { counts[n] = 4; needed[n++] = first; }
+    for (int h = 0; h < 2; h++) if (b_km && sb.half[h] == want) { counts[n] = 4; needed[n++] = first; }
   }
   int last = -1;
   for (int i = 0; i < n; i++)
@@ -476,12 +486,20 @@ constexpr int copies_in_flight(bool a_km, bool b_km, bool a_late, bool b_split, 
   for (int i = last + 1; i < n; i++) sum += counts[i];
   return sum;
 }
-static_assert(copies_in_flight(false, false, false, false, 0) == 16 && copies_in_flight(true, true, false, false, 1) == 0 &&
-              copies_in_flight(true, true, false, false, 0) == 16 && copies_in_flight(true, false, false, false, 1) == 4 &&
-              copies_in_flight(true, false, false, false, 0) == 16, "issue-order model");
+static_assert(copies_in_flight(false, false, {}, {}, false, 0) == 16 && copies_in_flight(true, true, {{1, 1}}, {{1, 1}}, false, 1) == 0 &&
+              copies_in_flight(true, true, {{1, 1}}, {{1, 1}}, false, 0) == 16 && copies_in_flight(true, false, {{1, 1}}, {}, false, 1) == 4 &&
+              copies_in_flight(true, false, {{1, 1}}, {}, false, 0) == 16 && copies_in_flight(true, true, {{0, 0}}, {{1, 1}}, false, 0) == 16 &&
+              copies_in_flight(true, true, {{0, 0}}, {{1, 1}}, false, 1) == 0 && copies_in_flight(false, false, {}, {}, true, 0) == 12,
+              "issue-order model");
 
-#ifndef LT_A_LATE
-#define LT_A_LATE 1
+#ifndef LT_NT_A
+#define LT_NT_A {0, 0}
+#endif
+#ifndef LT_NT_B
+#define LT_NT_B {2, 2}
+#endif
+#ifndef LT_NN_A
+#define LT_NN_A {0, 2}
 #endif
 #ifndef LT_B_SPLIT
 #define LT_B_SPLIT 1
@@ -568,23 +586,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   setup_a(0);
   setup_b(0);
   // copies of the unit that holds k-step t (a block for k-major operands) into the buffer of position I
-  auto copy_a = [&](auto steady, auto I, int t) {
+  auto copy_a = [&](auto steady, auto I, int t, auto J0, auto J1) {
     int seg = ca.seg;
     if constexpr (!decltype(steady)::value) {  // the steady loop never crosses a k-segment boundary
       seg = t >= kt_seg0;
       if (seg != ca.seg) setup_a(seg);
     }
     const int ks = rotated(seg ? t - kt_seg0 : t);
-    ca.template issue<K_TAIL>(A_KM ? ks >> 1 : ks, a_buf(I), wave, p.K[seg]);
+    ca.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(A_KM ? ks >> 1 : ks, a_buf(I), wave, p.K[seg]);
   };
-  auto copy_b = [&](auto steady, auto I, int t) {
+  auto copy_b = [&](auto steady, auto I, int t, auto J0, auto J1) {
     int seg = cb.seg;
     if constexpr (!decltype(steady)::value) {
       seg = t >= kt_seg0;
       if (seg != cb.seg) setup_b(seg);
     }
     const int ks = rotated(seg ? t - kt_seg0 : t);
-    cb.template issue<K_TAIL>(B_KM ? ks >> 1 : ks, b_buf(I), wave, p.K[seg]);
+    cb.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(B_KM ? ks >> 1 : ks, b_buf(I), wave, p.K[seg]);
   };
 
   // ---- MFMA operand fragments: 8 k values of row / column lane % 32 of a 32-wide block
@@ -632,49 +650,69 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   //                   matrix instructions on the second 16 k
   // I = t mod 4 at compile time.  steady == true: straight-line code, valid while every copy it issues exists and stays
   // inside the current k-segment.
-  // Copies are spread over the half-steps so that the address unit, which the four wavefronts share, is not handed a
-  // whole block at once: a k-major A block goes out in the second half of odd k-steps (A_LATE), mn-major B in the second
-  // half of every k-step (B_SPLIT); the rest in the first half.
-  constexpr bool A_LATE = A_KM && LT_A_LATE, B_SPLIT = !B_KM && !A_KM && LT_B_SPLIT;
+  // Copies are spread over the half-steps so that the address unit, which the four wavefronts share, is not handed whole
+  // blocks at once: the halves of a k-major block go out in the slots of SA / SB, mn-major B (next to mn-major A) in the
+  // second half of every k-step (B_SPLIT); the rest in the first half.
+  constexpr BlockSlots SA = B_KM ? BlockSlots{LT_NT_A} : BlockSlots{LT_NN_A}, SB = BlockSlots{LT_NT_B};
+  constexpr bool B_SPLIT = !B_KM && !A_KM && LT_B_SPLIT;
+  using J0 = std::integral_constant<int, 0>;
+  using J4 = std::integral_constant<int, 4>;
+  using J8 = std::integral_constant<int, 8>;
+  // the halves of the k-major blocks assigned to `slot`, for the block that starts at k-step t, into position I
+  auto copy_block_halves = [&](auto steady, auto slot, auto I, int t) {
+    constexpr int SLOT = decltype(slot)::value;
+    if constexpr (A_KM && SA.half[0] == SLOT) copy_a(steady, I, t, J0{}, J4{});
+    if constexpr (A_KM && SA.half[1] == SLOT) copy_a(steady, I, t, J4{}, J8{});
+    if constexpr (B_KM && SB.half[0] == SLOT) copy_b(steady, I, t, J0{}, J4{});
+    if constexpr (B_KM && SB.half[1] == SLOT) copy_b(steady, I, t, J4{}, J8{});
+  };
+  auto slot_copies = [&](int slot) constexpr {
+    return (A_KM ? 4 * ((SA.half[0] == slot) + (SA.half[1] == slot)) : 0) +
+           (B_KM ? 4 * ((SB.half[0] == slot) + (SB.half[1] == slot)) : 0);
+  };
   auto first_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
     load_frags(I, 1, af[1], bfr[1]);
     if (STEADY || t + 3 < kt_total) {  // mn-major: k-step t + 3 into the tile freed by the last barrier
-      if constexpr (!A_KM) copy_a(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
-      if constexpr (!B_KM && !B_SPLIT) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+      if constexpr (!A_KM) copy_a(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3, J0{}, J4{});
+      if constexpr (!B_KM && !B_SPLIT) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3, J0{}, J4{});
     }
     if constexpr ((i & 1) == 0 && N_KM > 0) {  // k-major: the block of k-steps t + 2, t + 3 into the other buffer
-      if (STEADY || t + 2 < kt_total) {
-        if constexpr (A_KM && !A_LATE) copy_a(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
-        if constexpr (B_KM) copy_b(steady, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
-      }
+      if (STEADY || t + 2 < kt_total)
+        copy_block_halves(steady, std::integral_constant<int, 1>{}, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
     }
 #pragma unroll
     for (int x = 0; x < FM; x++)
 #pragma unroll
       for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][x], bfr[0][y], acc[x][y], 0, 0, 0);
-    constexpr int COPIES = (A_KM ? 0 : 4) + ((B_KM || B_SPLIT) ? 0 : 4) +
-                           ((i & 1) == 0 ? ((A_KM && !A_LATE) ? 8 : 0) + (B_KM ? 8 : 0) : 0);
+    constexpr int COPIES = (A_KM ? 0 : 4) + ((B_KM || B_SPLIT) ? 0 : 4) + ((i & 1) == 0 ? slot_copies(1) : 0);
     SchedInterleave3<FRAG_READS, COPIES, FM * FN>::run();
   };
   auto second_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
-    constexpr int IN_FLIGHT = copies_in_flight(A_KM, B_KM, A_LATE, B_SPLIT, i & 1);
+    constexpr int IN_FLIGHT = copies_in_flight(A_KM, B_KM, SA, SB, B_SPLIT, i & 1);
     if constexpr (STEADY) wait_copies_and_barrier<IN_FLIGHT>();
     else wait_copies_and_barrier<0>();
     if (STEADY || t + 1 < kt_total) load_frags(std::integral_constant<int, (i + 1) & 3>{}, 0, af[0], bfr[0]);
-    if (STEADY || t + 3 < kt_total) {
-      // the barrier above freed the buffers of k-step t - 1 and, on odd t, the k-major buffer of k-steps t - 1, t
-      if constexpr (B_SPLIT) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
-      if constexpr (A_LATE && (i & 1) == 1) copy_a(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+    // the barrier above freed the buffers of k-step t - 1 and, on odd t, the k-major buffer of k-steps t - 1, t
+    if constexpr (B_SPLIT) {
+      if (STEADY || t + 3 < kt_total) copy_b(steady, std::integral_constant<int, (i + 3) & 3>{}, t + 3, J0{}, J4{});
+    }
+    if constexpr (N_KM > 0 && (i & 1) == 1) {
+      if (STEADY || t + 3 < kt_total)
+        copy_block_halves(steady, std::integral_constant<int, 0>{}, std::integral_constant<int, (i + 3) & 3>{}, t + 3);
+    }
+    if constexpr (N_KM > 0 && (i & 1) == 0) {
+      if (STEADY || t + 2 < kt_total)
+        copy_block_halves(steady, std::integral_constant<int, 2>{}, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
     }
 #pragma unroll
     for (int x = 0; x < FM; x++)
 #pragma unroll
       for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][x], bfr[1][y], acc[x][y], 0, 0, 0);
-    constexpr int COPIES = (B_SPLIT ? 4 : 0) + ((A_LATE && (i & 1) == 1) ? 8 : 0);
+    constexpr int COPIES = (B_SPLIT ? 4 : 0) + (N_KM > 0 ? slot_copies((i & 1) ? 0 : 2) : 0);
     SchedInterleave3<FRAG_READS, COPIES, FM * FN>::run();
   };
   using Steady = std::integral_constant<bool, true>;
@@ -684,19 +722,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   using P2 = std::integral_constant<int, 2>;
   using P3 = std::integral_constant<int, 3>;
 
-  // ---- prologue: k-steps 0..2 (k-major: block 0) in flight and landed, first half of k-step 0 issued
-  if constexpr (A_KM) copy_a(Ragged{}, P0{}, 0);
-  if constexpr (B_KM) copy_b(Ragged{}, P0{}, 0);
-  if constexpr (!A_KM) copy_a(Ragged{}, P0{}, 0);
-  if constexpr (!B_KM) copy_b(Ragged{}, P0{}, 0);
+  // ---- prologue: k-steps 0..2 (k-major: block 0 and the slot-0 halves of block 1) in flight and landed, first half of
+  //      k-step 0 issued
+  if constexpr (A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J8{});
+  if constexpr (B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J8{});
+  if constexpr (!A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J4{});
+  if constexpr (!B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J4{});
   if (kt_total > 1) {
-    if constexpr (!A_KM) copy_a(Ragged{}, P1{}, 1);
-    if constexpr (!B_KM) copy_b(Ragged{}, P1{}, 1);
+    if constexpr (!A_KM) copy_a(Ragged{}, P1{}, 1, J0{}, J4{});
+    if constexpr (!B_KM) copy_b(Ragged{}, P1{}, 1, J0{}, J4{});
   }
   if (kt_total > 2) {
-    if constexpr (!A_KM) copy_a(Ragged{}, P2{}, 2);
-    if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2);
-    if constexpr (A_LATE) copy_a(Ragged{}, P2{}, 2);  // the second block; later ones follow from the odd k-steps
+    if constexpr (!A_KM) copy_a(Ragged{}, P2{}, 2, J0{}, J4{});
+    if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2, J0{}, J4{});
+    if constexpr (N_KM > 0) copy_block_halves(Ragged{}, std::integral_constant<int, 0>{}, P2{}, 2);
   }
   wait_copies_and_barrier<0>();
   load_frags(P0{}, 0, af[0], bfr[0]);
