@@ -135,6 +135,8 @@ void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, 
   s.colsum_bytes = lt_colsum_workspace(T, lin.out_features);
   s.colsum = ws.take(s.colsum_bytes);
   s.skinny_bytes = lin.lowrank > 0 ? lt_gemm_skinny_workspace(T, lin.lowrank) : 0;
+  if (lin.block == 0 && dtype == LT_BF16)  // dW of a small dense layer: reduction over the tokens split across workgroups
+    s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_splitk_workspace(lin.out_features, lin.in_features, T));
   s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 
@@ -184,7 +186,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.A[0] = operand(dy, out, false);
       p.B[0] = operand(x_act, in, false);
       p.epi = epi_store_params(grads.weight, in, dtype, nullptr);
-      LT_TRY(lt_launch_gemm(p, EPI_STORE, dtype, io_dtype, stream));
+      LT_TRY(lt_launch_gemm_skinny(p, dtype, io_dtype, s.skinny, s.skinny_bytes, stream));
     } else {
       p.M = lin.block; p.N = in; p.K[0] = T;
       p.sp.mode = SPARSE_DW; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;

@@ -548,8 +548,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  const int kt_seg0 = (int)((p.K[0] + DK - 1) / DK);
-  const int kt_total = kt_seg0 + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
+  const int kt_all = (int)((p.K[0] + DK - 1) / DK) + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
+  // split-k (one k-segment only): this workgroup walks k-steps [kt_begin, kt_begin + kt_total) of kt_all; the slices are
+  // an even number of k-steps long so that k-major blocks stay whole.  Below, k-step numbers are local to the slice.
+  int kt_begin = 0, kt_total = kt_all;
+  if (p.ksplit > 1) {
+    const int per = (((kt_all + p.ksplit - 1) / p.ksplit) + 1) & ~1;
+    kt_begin = min(kt_all, (int)blockIdx.y * per);
+    kt_total = min(per, kt_all - kt_begin);
+  }
+  const int kt_seg0 = p.nseg > 1 ? (int)((p.K[0] + DK - 1) / DK) : kt_total;
 
   // ---- buffer of k-step position I (k-step index mod 4) and copy targets, selected at compile time
   auto a_buf = [&](auto I) -> bf16* {
@@ -569,15 +577,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   // differs between XCDs.  Measured on the up- and down-projection shapes: +16 % and +25 % for two k-major operands,
   // nothing to gain for mn-major ones.
   int rot = 0;
-  if (!K_TAIL && p.nseg == 1 && (kt_total & 1) == 0 && p.krot) {
+  if (!K_TAIL && p.nseg == 1 && (kt_all & 1) == 0 && p.krot) {
     const unsigned bx = blockIdx.x;
-    const unsigned r = (bx & 7) * (kt_total >> 3) +
-                       (p.krot == 1 ? ((bx >> 3) & 3) * (kt_total >> 5) : ((bx >> 3) & 7) * (kt_total >> 6));
-    rot = __builtin_amdgcn_readfirstlane((int)((r % (unsigned)kt_total) & ~1u));
+    const unsigned r = (bx & 7) * (kt_all >> 3) +
+                       (p.krot == 1 ? ((bx >> 3) & 3) * (kt_all >> 5) : ((bx >> 3) & 7) * (kt_all >> 6));
+    rot = __builtin_amdgcn_readfirstlane((int)((r % (unsigned)kt_all) & ~1u));
   }
   auto rotated = [&](int ks) {
     const int r = ks + rot;
-    return r >= kt_total ? r - kt_total : r;
+    return r >= kt_all ? r - kt_all : r;
   };
   DmaOperand<A_KM> ca;
   DmaOperand<B_KM> cb;
@@ -592,7 +600,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       seg = t >= kt_seg0;
       if (seg != ca.seg) setup_a(seg);
     }
-    const int ks = rotated(seg ? t - kt_seg0 : t);
+    const int ks = rotated(seg ? t - kt_seg0 : t + kt_begin);
     ca.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(A_KM ? ks >> 1 : ks, a_buf(I), wave, p.K[seg]);
   };
   auto copy_b = [&](auto steady, auto I, int t, auto J0, auto J1) {
@@ -601,7 +609,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       seg = t >= kt_seg0;
       if (seg != cb.seg) setup_b(seg);
     }
-    const int ks = rotated(seg ? t - kt_seg0 : t);
+    const int ks = rotated(seg ? t - kt_seg0 : t + kt_begin);
     cb.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(B_KM ? ks >> 1 : ks, b_buf(I), wave, p.K[seg]);
   };
 
@@ -776,6 +784,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   //      consecutive columns per lane, so that the fused epilogue reads and writes HBM in 16-byte pieces of contiguous rows.
   //      Staged column c of row r sits at c ^ 32 when bit 2 of r is set: the two half-waves of a transposing write (rows
   //      r and r + 4, same columns) then hit different banks without padding the rows.
+  EpiParams epi = p.epi;
+  if (KIND == EPI_STORE && p.ksplit > 1) epi.out = reinterpret_cast<float*>(epi.out) + (int64_t)blockIdx.y * p.split_stride;
   float* stage = reinterpret_cast<float*>(wave == 0   ? (A_KM ? a_d0 : a_s0)
                                           : wave == 1 ? (A_KM ? a_d1 : a_s1)
                                           : wave == 2 ? (B_KM ? b_d0 : b_s0)
@@ -805,7 +815,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
           vg[e] = sg[e];
           vl[e] = sl[e];
         }
-        if (m < p.M) epi_act_fwd_gated8(p.epi, m, n0 + wn * (WTN / 2) + c, vg, vl);
+        if (m < p.M) epi_act_fwd_gated8(epi, m, n0 + wn * (WTN / 2) + c, vg, vl);
       }
     } else {
       constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
@@ -813,22 +823,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       const int64_t n = n0 + wn * WTN + c;
       const int64_t mlane = mrow0 + lane / LANES_PER_ROW;  // this lane's row in iteration 0
       // global reads of the epilogue run two iterations ahead of their use
-      EpiLoad l0 = epi_load8<KIND, TX>(p.epi, mlane, n, mlane < p.M);
-      EpiLoad l1 = epi_load8<KIND, TX>(p.epi, mlane + ROWS_PER_IT, n, mlane + ROWS_PER_IT < p.M);
+      EpiLoad l0 = epi_load8<KIND, TX>(epi, mlane, n, mlane < p.M);
+      EpiLoad l1 = epi_load8<KIND, TX>(epi, mlane + ROWS_PER_IT, n, mlane + ROWS_PER_IT < p.M);
       for (int it = 0; it < NIT; it++) {
         const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
         const int64_t m = mrow0 + row;
         const int64_t m2 = m + 2 * ROWS_PER_IT;
-        const EpiLoad l2 = epi_load8<KIND, TX>(p.epi, m2, n, it + 2 < NIT && m2 < p.M);
+        const EpiLoad l2 = epi_load8<KIND, TX>(epi, m2, n, it + 2 < NIT && m2 < p.M);
         float v[8];
         const float* sv = staged(row, c);
 #pragma unroll
         for (int e = 0; e < 8; e++) v[e] = sv[e];
         if (m < p.M) {
-          if constexpr (KIND == EPI_STORE) epi_store8(p.epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(p.epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(p.epi, m, n, v, l0);
-          else epi_out8_loaded<TX>(p.epi, m, n, v, l0);
+          if constexpr (KIND == EPI_STORE) epi_store8(epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(epi, m, n, v, l0);
+          else epi_out8_loaded<TX>(epi, m, n, v, l0);
         }
         l0 = l1;
         l1 = l2;
@@ -849,7 +859,7 @@ int launch_dma(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
   const int tiles_n = (int)(p.N / (gated ? 128 : 256));
   bool k_tail = false;
   for (int s = 0; s < p.nseg; s++) k_tail = k_tail || (p.K[s] % DK != 0);
-  dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(p.ksplit > 1 ? p.ksplit : 1)), block(256);
   const bool bf16_io = KIND == EPI_OUT && io_dtype == LT_BF16;
   if constexpr (!A_KM && !B_KM) {
     if (k_tail) {
@@ -871,7 +881,7 @@ int launch_cfg(const GemmProblem& p, int io_dtype, hipStream_t stream) {
   const bool gated = KIND == EPI_ACT_FWD && p.epi.gated;
   const int tiles_m = (int)((p.M + BM - 1) / BM);
   const int tiles_n = (int)(p.N / (gated ? BN / 2 : BN));
-  dim3 grid((unsigned)(tiles_m * tiles_n)), block(WM * WN * 64);
+  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(p.ksplit > 1 ? p.ksplit : 1)), block(WM * WN * 64);
   if (KIND == EPI_OUT && io_dtype == LT_BF16) {
     hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, WM, WN, A_KM, B_KM, KIND, bf16>), grid, block, 0, stream, p, tiles_m,
                        tiles_n);
@@ -1019,6 +1029,22 @@ size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank) {
   return lt_align_up((size_t)SKINNY_MAX_SLICES * (size_t)tokens * (size_t)lowrank * sizeof(float), 256);
 }
 
+namespace {
+// slices of the reduction for an [M, N] result on 256 x 256 tiles: enough workgroups for the 256 CUs, each slice at least
+// 16 k-steps long
+int splitk_slices(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (tiles >= 128) return 1;
+  const int64_t by_k = K / (16 * DK);
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, by_k), 8));
+}
+}  // namespace
+
+size_t lt_gemm_splitk_workspace(int64_t M, int64_t N, int64_t K) {
+  const int slices = splitk_slices(M, N, K);
+  return slices > 1 ? lt_align_up((size_t)slices * (size_t)M * (size_t)N * sizeof(float), 256) : 0;
+}
+
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                           hipStream_t stream) {
   const bool a_km = p.A[0].kmajor, b_km = p.B[0].kmajor;
@@ -1027,9 +1053,25 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
             !(!a_km && b_km) && (a_km || p.M % 128 == 0) && ((!a_km && !b_km) || p.K[0] % BK == 0) && p.K[0] > 0 &&
             p.A[0].ld % 8 == 0 && p.B[0].ld % 8 == 0 && lt_aligned(p.A[0].ptr, 16) && lt_aligned(p.B[0].ptr, 16) &&
             e.ldo == p.N && lt_aligned(e.out, 16) && (!e.bias || lt_aligned(e.bias, 16));
-  // shapes the 256 x 256 kernels fill the chip with keep going there
   const int64_t tiles = ((p.M + 127) / 128) * (p.N / 128);
-  if (ok && lt_gemm_mfma_supported(p, EPI_STORE) && ((p.M + 255) / 256) * (p.N / 256) >= 128) ok = false;
+  if (dtype == LT_BF16 && p.sp.mode == SPARSE_NONE && lt_gemm_mfma_supported(p, EPI_STORE)) {
+    // 256 x 256 tiles fit: the copy-based kernel, its reduction split when the tiles alone leave CUs idle
+    const int slices = p.nseg == 1 ? splitk_slices(p.M, p.N, p.K[0]) : 1;
+    const size_t need = (size_t)slices * (size_t)p.M * (size_t)p.N * sizeof(float);
+    if (slices > 1 && workspace && workspace_bytes >= need && g_mfma_variant != 1 && p.K[0] % 64 == 0 && e.ldo == p.N &&
+        dma_offsets_fit(p, EPI_STORE)) {
+      GemmProblem q = p;
+      q.ksplit = slices;
+      q.split_stride = p.M * p.N;
+      q.epi.out = workspace;
+      q.epi.ldo = p.N;
+      q.epi.out_dtype = LT_F32;
+      q.epi.bias = nullptr;
+      LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+      return lt_splitk_reduce((const float*)workspace, slices, p.M * p.N, p.M * p.N, (int)p.N, e.bias, e.out_dtype, e.out, stream);
+    }
+    if (((p.M + 255) / 256) * (p.N / 256) >= 64 || slices == 1) ok = false;
+  }
   if (!ok) return lt_launch_gemm(p, EPI_STORE, dtype, io_dtype, stream);
   const int kt_total = (int)((p.K[0] + BK - 1) / BK);
   int slices = 1;

@@ -341,6 +341,8 @@ int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtyp
 // 128 x 128 tiles, the reduction split over workgroups through `workspace` when that fills the chip better.  Falls back to
 // lt_launch_gemm when the shape does not fit.
 size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank);
+// partial sums of a split [M, N] result on 256 x 256 tiles (0 when the tiles alone fill the chip)
+size_t lt_gemm_splitk_workspace(int64_t M, int64_t N, int64_t K);
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                           hipStream_t stream);
 // out[i] = sum_s partial[s * stride + i] (+ bias[i % cols]) for i < count, cast to out_dtype

@@ -330,6 +330,14 @@ def test_config3_bf16_full_size_headline():
     _full_size_checks(ffn, x, dy, 0.0)
 
 
+def test_config5_layer_shape_bf16_split_reduction():
+    """one FFN layer at BASELINE config 5's shape (hidden 768, intermediate 3072, GeGLU, 16 x 1024 tokens): the weight
+    gradients are [6144, 768] and [768, 3072], too few 256 x 256 tiles for 256 CUs, so their reduction over the tokens is
+    split across workgroups and summed from fp32 partial results"""
+    ffn, x, dy = _headline(768, 3072, True, 0.02, 0.0, (16, 1024))
+    _full_size_checks(ffn, x, dy, 0.0)
+
+
 @pytest.mark.parametrize("stretch", [True, False])
 def test_config4_pixelfly_bf16_full_size(stretch):
     """BASELINE config 4: config 3's shape with PixelFly block-sparse projections (64 x 64 blocks, 7 of 64 blocks per block
