@@ -184,6 +184,11 @@ def main():
                      **({"tflops": fl / (ms * 1e-3) / 1e12} if fl > 0 else {}),
                      **({"gbps": by / (ms * 1e-3) / 1e9} if by > 0 else {})} for name, n, ms, fl, by in kernels]
 
+    # L2 <-> memory bytes per GEMM launch (fetch + write, averaged over the six launches of a step), from the FETCH_SIZE
+    # and WRITE_SIZE counter runs of this command summarised in profiles/leanffn_config3_gemm_hbm_traffic.txt
+    # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration on the dy cast kernel); only measured for config 3
+    traffic = 1.588e9 if args.config == "c3" else None
+
     result = {
         "metric": METRIC, "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -193,7 +198,7 @@ def main():
         "tflops": tflops, "mfma_util_pct": 100.0 * tflops / peak,
         "peak_activation_mb": peak_mb, "saved_activation_mb": saved_mb,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                     "frac": achieved / peak, "traffic": None,
+                     "frac": achieved / peak, "traffic": traffic,
                      "kernel": "all GEMM launches of a step: " + ", ".join(sorted({k[0] for k in gemm})),
                      "flops_per_launch": gemm_flops / max(gemm_launches, 1),
                      "avg_launch_us": gemm_ms / max(gemm_launches, 1) * 1e3},
