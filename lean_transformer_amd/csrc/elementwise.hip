@@ -646,3 +646,11 @@ int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t c
   LT_LAUNCH_CHECK();
   return LT_OK;
 }
+
+int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream) {
+  LT_REQUIRE(rows > 0 && cols > 0 && partial && out, LT_ERR_BAD_ARG, "colreduce: bad arguments");
+  LtProfileScope scope("colreduce", 0.0, (double)cols * 4.0 * (rows + 1), stream);
+  hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(cols, 256)), dim3(256), 0, stream, rows, stride, cols, partial, out);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}

@@ -143,9 +143,12 @@ void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, 
 // gradient side of one generalized linear layer.  The input-gradient GEMM runs FIRST, through epilogue `kind_dx`
 // (EPI_ACT_BWD for the down-projection, whose epilogue also re-materialises this layer's own input `x_act`), then the
 // parameter gradients, which may therefore read x_act.  Pass kind_dx < 0 to skip the input gradient.
+// act_colsum / act_colsum_done: with an EPI_ACT_BWD input-gradient epilogue, room for the partial column sums of the dpre it
+// writes (one row of epi_dx.ld_pre floats per 128 tokens); *act_colsum_done says whether the kernel that ran filled it
 int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void* x_act, const void* dy,
                          const void* lowrank_hid, int kind_dx, const EpiParams& epi_dx, const lt_linear_grads& grads,
-                         const LinearBwdScratch& s, int io_dtype, hipStream_t stream) {
+                         const LinearBwdScratch& s, int io_dtype, hipStream_t stream, float* act_colsum = nullptr,
+                         bool* act_colsum_done = nullptr) {
   const int64_t in = lin.in_features, out = lin.out_features, r = lin.lowrank;
   const bool need_dx = kind_dx >= 0;
   if (r > 0 && (need_dx || grads.lowrank_first)) {  // g_hid = dy L2  [T, r]
@@ -169,6 +172,10 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.K[0] = out;
       p.A[0] = operand(dy, out, true);
       p.B[0] = operand(lin.weight, in, false);
+      if (kind_dx == EPI_ACT_BWD && act_colsum && lt_gemm_fuses_colsum(p, dtype, io_dtype)) {
+        p.epi.colsum = act_colsum;
+        *act_colsum_done = true;
+      }
       LT_TRY(lt_launch_gemm(p, kind_dx, dtype, io_dtype, stream));
     } else {
       p.K[0] = lin.block;
@@ -263,6 +270,7 @@ struct BwdScratch {
   float* du;         // [T, H] fp32
   void* ln_ws;
   size_t ln_ws_bytes;
+  float* act_colsum;  // [ceil(T / 128), N1]: partial column sums of dpre from the epilogue that writes it
   LinearBwdScratch h2o, i2h;
 };
 
@@ -279,6 +287,7 @@ void plan_backward(const lt_ffn_desc& d, Bump& ws, BwdScratch& s) {
   s.du = (float*)ws.take((size_t)T * d.hidden * sizeof(float));
   s.ln_ws_bytes = lt_ln_backward_workspace(T, d.hidden);
   s.ln_ws = ws.take(s.ln_ws_bytes);
+  s.act_colsum = (float*)ws.take((size_t)((T + 127) / 128) * n1 * sizeof(float));
   plan_linear_backward(d.h2o, T, d.compute_dtype, ws, s.h2o);
   plan_linear_backward(d.i2h, T, d.compute_dtype, ws, s.i2h);
 }
@@ -388,13 +397,19 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   }
 
   // down-projection backward; its input-gradient epilogue turns dh into dP and re-materialises h from P
+  bool bias_from_epilogue = false;
   {
     EpiParams e;
     memset(&e, 0, sizeof(e));
     e.pre = saved->pre_activation; e.ld_pre = N1; e.dpre = s.dpre; e.hid = s.hid; e.ld_hid = I;
     e.gated = d.gated; e.act = d.act; e.inter = I;
     LT_TRY(linear_backward_impl(d.h2o, T, cdt, s.hid, g, saved->h2o_lowrank_hid, EPI_ACT_BWD, e, grads->h2o, s.h2o, io,
-                                stream));
+                                stream, grads->i2h.bias ? s.act_colsum : nullptr, &bias_from_epilogue));
+  }
+  lt_linear_grads i2h_grads = grads->i2h;
+  if (bias_from_epilogue) {  // db1 = column sums of dP, already reduced to one row per 128 tokens
+    LT_TRY(lt_colreduce((int)((T + 127) / 128), N1, (int)N1, s.act_colsum, (float*)grads->i2h.bias, stream));
+    i2h_grads.bias = nullptr;
   }
 
   // up-projection backward on the recomputed LayerNorm output; du in fp32
@@ -404,7 +419,7 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   {
     EpiParams e = epi_store_params(s.du, H, LT_F32, nullptr);
     LT_TRY(linear_backward_impl(d.i2h, T, cdt, s.u, s.dpre, saved->i2h_lowrank_hid, need_du ? EPI_STORE : -1, e,
-                                grads->i2h, s.i2h, io, stream));
+                                i2h_grads, s.i2h, io, stream));
   }
   if (need_du) {
     LT_TRY(lt_ln_backward(T, (int)H, io, x, saved->ln_stats, d.ln_weight, LT_F32, s.du, io, d.residual ? dy : nullptr,

@@ -793,6 +793,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   static_assert(32 * WTN * 4 <= MN_ELEMS * 2, "a 32-row strip must fit the smallest buffer");
   auto staged = [&](int row, int col) -> float* { return &stage[row * WTN + (col ^ (((row >> 2) & 1) << 5))]; };
   const bool pair = (KIND == EPI_ACT_FWD) && gated;
+  float colsum[16];  // EPI_ACT_BWD: column sums of this lane's 8 (+ 8) dpre columns over the rows it writes
+#pragma unroll
+  for (int e = 0; e < 16; e++) colsum[e] = 0.f;
 #pragma unroll
   for (int i = 0; i < FM; i++) {
 #pragma unroll
@@ -837,7 +840,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
         if (m < p.M) {
           if constexpr (KIND == EPI_STORE) epi_store8(epi, m, n, v);
           else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(epi, m, n, v, l0);
+          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(epi, m, n, v, l0, colsum);
           else epi_out8_loaded<TX>(epi, m, n, v, l0);
         }
         l0 = l1;
@@ -845,6 +848,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       }
     }
     __builtin_amdgcn_wave_barrier();
+  }
+  if constexpr (KIND == EPI_ACT_BWD) {
+    if (epi.colsum) {
+      // lanes l, l + 16, l + 32, l + 48 hold the same columns for different rows of the wavefront's 128-row sub-tile
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        colsum[e] += __shfl_xor(colsum[e], 16);
+        colsum[e] += __shfl_xor(colsum[e], 32);
+      }
+      if (lane < 16) {
+        float* dst = epi.colsum + ((m0 + wm * WTM) / 128) * epi.ld_pre + n0 + wn * WTN + lane * 8;
+        float lo[8], hi[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          lo[e] = colsum[e];
+          hi[e] = colsum[8 + e];
+        }
+        store8(dst, lo);
+        if (epi.gated) store8(dst + epi.inter, hi);
+      }
+    }
   }
 }
 
@@ -933,15 +957,21 @@ bool dma_offsets_fit(const GemmProblem& p, int kind) {
 
 int g_mfma_variant = 0;  // 0: choose; 1: register-staged kernel; 2: copy-based kernel (tests and benchmarks)
 
-template <bool A_KM, bool B_KM, int KIND> int launch_tile(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+// whether a problem the tiled kernels take goes to the copy-based one
+bool dma_selected(const GemmProblem& p, int kind, int io_dtype) {
+  const bool a_km = p.A[0].kmajor, b_km = p.B[0].kmajor;
   bool k_tail = false, k_blocks = true;
   for (int s = 0; s < p.nseg; s++) {
     k_tail = k_tail || (p.K[s] % DK != 0);
     k_blocks = k_blocks && (p.K[s] % 64 == 0);  // k-major operands are copied in whole blocks of 64 k
   }
-  const bool dma_ok = dma_offsets_fit(p, KIND) && !(k_tail && KIND == EPI_OUT && io_dtype == LT_BF16) &&
-                      ((!A_KM && !B_KM) || k_blocks);
-  if (g_mfma_variant != 1 && dma_ok) return launch_dma<A_KM, B_KM, KIND>(p, io_dtype, stream);
+  const bool dma_ok = dma_offsets_fit(p, kind) && !(k_tail && kind == EPI_OUT && io_dtype == LT_BF16) &&
+                      ((!a_km && !b_km) || k_blocks);
+  return g_mfma_variant != 1 && dma_ok;
+}
+
+template <bool A_KM, bool B_KM, int KIND> int launch_tile(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+  if (dma_selected(p, KIND, io_dtype)) return launch_dma<A_KM, B_KM, KIND>(p, io_dtype, stream);
   return launch_cfg<256, 256, 2, 2, A_KM, B_KM, KIND>(p, io_dtype, stream);
 }
 
@@ -982,6 +1012,11 @@ bool lt_gemm_mfma_supported(const GemmProblem& p, int kind) {
     if (!lt_aligned(p.A[s].ptr, 16) || !lt_aligned(p.B[s].ptr, 16)) return false;
   }
   return true;
+}
+
+bool lt_gemm_fuses_colsum(const GemmProblem& p, int dtype, int io_dtype) {
+  return dtype == LT_BF16 && p.sp.mode == SPARSE_NONE && lt_gemm_mfma_supported(p, EPI_ACT_BWD) &&
+         dma_selected(p, EPI_ACT_BWD, io_dtype) && p.epi.ld_pre % 8 == 0;
 }
 
 static const char* mfma_tag(const GemmProblem& p, int kind) {

@@ -32,6 +32,9 @@ struct EpiParams {
   int gated;
   int act;
   int64_t inter;      // I
+  // ACT_BWD on the copy-based kernel only (see lt_gemm_fuses_colsum): column sums of the dpre values as stored, one partial
+  // row per 128 rows of the output: colsum[(m / 128) * ld_pre + column].  Null = off.
+  float* colsum;
   // EPI_OUT
   const void* x;      // residual input [M, ldy] (null = no residual)
   void* y;            // [M, ldy]
@@ -268,8 +271,9 @@ __device__ __forceinline__ void unpack_bf16x8(const lt_u32x4& raw, float (&v)[8]
   for (int i = 0; i < 8; i++) v[i] = (float)t.h[i];
 }
 
+// cs: running column sums of the 8 gate-side (and, gated, 8 linear-side at cs + 8) dpre values this lane has written
 __device__ __forceinline__ void epi_act_bwd8_loaded(const EpiParams& e, int64_t m, int64_t n, const float (&dh)[8],
-                                                    const EpiLoad& l) {
+                                                    const EpiLoad& l, float (&cs)[16]) {
   bf16* dpre = reinterpret_cast<bf16*>(e.dpre) + m * e.ld_pre + n;
   float pg[8], a[8], da[8], o[8];
   unpack_bf16x8(l.a, pg);
@@ -282,14 +286,20 @@ __device__ __forceinline__ void epi_act_bwd8_loaded(const EpiParams& e, int64_t 
     for (int i = 0; i < 8; i++) o[i] = dh[i] * pl[i] * da[i];
     store8(dpre, o);
 #pragma unroll
+    for (int i = 0; i < 8; i++) cs[i] += (float)(bf16)o[i];
+#pragma unroll
     for (int i = 0; i < 8; i++) o[i] = dh[i] * a[i];
     store8(dpre + e.inter, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) cs[8 + i] += (float)(bf16)o[i];
 #pragma unroll
     for (int i = 0; i < 8; i++) a[i] *= pl[i];
   } else {
 #pragma unroll
     for (int i = 0; i < 8; i++) o[i] = dh[i] * da[i];
     store8(dpre, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) cs[i] += (float)(bf16)o[i];
   }
   if (e.hid) store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, a);
 }
@@ -343,6 +353,10 @@ int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtyp
 size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank);
 // partial sums of a split [M, N] result on 256 x 256 tiles (0 when the tiles alone fill the chip)
 size_t lt_gemm_splitk_workspace(int64_t M, int64_t N, int64_t K);
+// true when lt_launch_gemm sends this EPI_ACT_BWD problem to the kernel that fills EpiParams::colsum
+bool lt_gemm_fuses_colsum(const GemmProblem& p, int dtype, int io_dtype);
+// out[c] = sum over `rows` partial rows of partial[r * stride + c]
+int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream);
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                           hipStream_t stream);
 // out[i] = sum_s partial[s * stride + i] (+ bias[i % cols]) for i < count, cast to out_dtype

@@ -190,6 +190,8 @@ class _LeanFFN(torch.autograd.Function):
             ctx, tokens, hidden, ln_weight, ln_bias, i2h_weight, i2h_bias, i2h_lowrank_first, i2h_lowrank_second,
             i2h_forward_indices, i2h_backward_indices, h2o_weight, h2o_bias, h2o_lowrank_first, h2o_lowrank_second,
             h2o_forward_indices, h2o_backward_indices, post_ln_weight, post_ln_bias, io)
+        # fp32 copies of the small vectors (LayerNorm parameters, biases): backward reuses them instead of converting again
+        ctx._small_fp32 = (keep[0], keep[1], keep[2], keep[3], keep[4][1], keep[5][1])
         n1 = desc.i2h.out_features
         y = torch.empty_like(x)
         pre_activation = torch.empty(tokens, n1, dtype=cdt, device=device)
@@ -254,9 +256,10 @@ class _LeanFFN(torch.autograd.Function):
         if dy.dtype != io:
             dy = dy.to(io)
         dy = dy.contiguous()
+        ln_w32, ln_b32, post_w32, post_b32, i2h_b32, h2o_b32 = ctx._small_fp32
         desc, keep = _LeanFFN._describe(
-            ctx, tokens, hidden, ln_weight, ln_bias, i2h_weight, i2h_bias, i2h_l1, i2h_l2, i2h_fwd, i2h_bwd,
-            h2o_weight, h2o_bias, h2o_l1, h2o_l2, h2o_fwd, h2o_bwd, post_ln_weight, post_ln_bias, io)
+            ctx, tokens, hidden, ln_w32, ln_b32, i2h_weight, i2h_b32, i2h_l1, i2h_l2, i2h_fwd, i2h_bwd,
+            h2o_weight, h2o_b32, h2o_l1, h2o_l2, h2o_fwd, h2o_bwd, post_w32, post_b32, io)
         need = ctx.needs_input_grad
 
         def new(like_shape, dtype, wanted):
@@ -265,14 +268,25 @@ class _LeanFFN(torch.autograd.Function):
         need_ln = need[1] or need[2]
         need_post = post_ln_weight is not None and (need[17] or need[18])
         dx = new(x.shape, io, need[0])
-        d_ln_w, d_ln_b = new((hidden,), torch.float32, need_ln), new((hidden,), torch.float32, need_ln)
-        d_post_w, d_post_b = new((hidden,), torch.float32, need_post), new((hidden,), torch.float32, need_post)
+        # the kernels write the gradients of the small vectors in fp32: they share one buffer (256-byte aligned pieces) so
+        # that a single conversion brings them to the parameters' dtype afterwards
+        small_sizes = [hidden if need_ln else 0, hidden if need_ln else 0, hidden if need_post else 0,
+                       hidden if need_post else 0, desc.i2h.out_features if i2h_bias is not None and need[4] else 0,
+                       hidden if h2o_bias is not None and need[11] else 0]
+        small_offsets, total = [], 0
+        for n in small_sizes:
+            small_offsets.append(total)
+            total += -(-n // 64) * 64
+        small = torch.empty(total, dtype=torch.float32, device=device)
+
+        def piece(buffer, i):
+            return buffer[small_offsets[i]:small_offsets[i] + small_sizes[i]] if small_sizes[i] else None
+
+        d_ln_w, d_ln_b, d_post_w, d_post_b, d_i2h_b, d_h2o_b = (piece(small, i) for i in range(6))
         d_i2h_w = new(i2h_weight.shape, cdt, need[3])
-        d_i2h_b = new((desc.i2h.out_features,), torch.float32, i2h_bias is not None and need[4])
         d_i2h_l1 = new(i2h_l1.shape, cdt, need[5]) if i2h_l1 is not None else None
         d_i2h_l2 = new(i2h_l2.shape, cdt, need[6]) if i2h_l2 is not None else None
         d_h2o_w = new(h2o_weight.shape, cdt, need[10])
-        d_h2o_b = new((hidden,), torch.float32, h2o_bias is not None and need[11])
         d_h2o_l1 = new(h2o_l1.shape, cdt, need[12]) if h2o_l1 is not None else None
         d_h2o_l2 = new(h2o_l2.shape, cdt, need[13]) if h2o_l2 is not None else None
         outputs = (dx, d_ln_w, d_ln_b, d_post_w, d_post_b, d_i2h_w, d_i2h_b, d_i2h_l1, d_i2h_l2, d_h2o_w, d_h2o_b,
@@ -294,6 +308,11 @@ class _LeanFFN(torch.autograd.Function):
             for g in outputs[1:]:
                 if g is not None:
                     g.zero_()
+        small_params = (ln_weight, ln_bias, post_ln_weight, post_ln_bias, i2h_bias, h2o_bias)
+        wanted = {t.dtype for t, n in zip(small_params, small_sizes) if n}
+        if len(wanted) == 1 and wanted != {torch.float32} and total:
+            converted = small.to(wanted.pop())
+            d_ln_w, d_ln_b, d_post_w, d_post_b, d_i2h_b, d_h2o_b = (piece(converted, i) for i in range(6))
         grad_input = None if dx is None else dx.view(*input.shape)
         return (grad_input, d_ln_w if need[1] else None, d_ln_b if need[2] else None,
                 d_i2h_w, d_i2h_b, d_i2h_l1, d_i2h_l2, None, None, None,
