@@ -6,7 +6,8 @@
 //
 // Work decomposition: 256 threads = 4 wavefronts in a 2 x 2 grid over a 128 x 128 output tile; each wavefront owns a
 // 64 x 64 quadrant as 2 x 2 MFMA blocks of 32 x 32.  Operand tiles of 16 k-steps are converted to fp32 on load and staged
-// in LDS k-major ([k][row], padded by 4 floats so the 32 rows x 2 k-lanes of one MFMA operand read conflict-free).
+// in LDS k-major ([k][row], padded by 4 floats so the 32 rows x 2 k-lanes of one MFMA operand read conflict-free); the loads
+// of the next step are in flight (in registers) while the matrix cores work on the current one.
 #include "lt_gemm.h"
 
 namespace {
@@ -22,8 +23,8 @@ template <typename TI> struct Segment {
 
 template <typename TI, int KIND, typename TC, typename TX>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmProblem p) {
-  __shared__ float As[GBK][GBM + GPAD];
-  __shared__ float Bs[GBK][GBN + GPAD];
+  __shared__ __attribute__((aligned(16))) float As[2][GBK][GBM + GPAD];
+  __shared__ __attribute__((aligned(16))) float Bs[2][GBK][GBN + GPAD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const bool gated = (KIND == EPI_ACT_FWD) && p.epi.gated;
@@ -101,52 +102,126 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmProblem p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  for (int seg = 0; seg < nseg; seg++) {
-    const Segment<TI> g = segment(seg);
-    for (int64_t k0 = 0; k0 < g.K; k0 += GBK) {
-      // ---- stage one 128 x 16 tile of each operand, 8 elements per thread, threads adjacent along the contiguous axis
+  // ---- main loop, software-pipelined: the 128 x 16 operand tiles of step i + 1 are fetched into registers (two 4-element
+  //      vectors per operand and thread, along the contiguous axis; element by element where alignment or bounds do not
+  //      allow vectors) while the matrix cores work on step i out of LDS; two LDS buffers, one barrier per step.
+  struct Fetch {
+    float a[2][4], b[2][4];
+  };
+  int seg = 0;
+  Segment<TI> g = segment(0);
+  int64_t k0 = 0;
+  auto fetch = [&](Fetch& f) {
+    // A: k-major -> 4 consecutive k of one row; mn-major -> 4 consecutive rows of one k
+    const bool va = (reinterpret_cast<uintptr_t>(g.A) % (4 * sizeof(TI)) == 0) && (g.lda & 3) == 0 &&
+                    (g.a_km ? (g.K & 3) == 0 : (M & 3) == 0);
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        int kk, mm;
-        if (g.a_km) { kk = tid & 15; mm = (tid >> 4) + i * 16; } else { mm = tid & 127; kk = (tid >> 7) + i * 2; }
-        const int64_t gm = m0 + mm, gk = k0 + kk;
-        float v = 0.f;
-        if (gm < M && gk < g.K) v = g.a_km ? ldf(g.A, gm * g.lda + gk) : ldf(g.A, gk * g.lda + gm);
-        As[kk][mm] = v;
-      }
+    for (int i = 0; i < 2; i++) {
+      int kk, mm;
+      if (g.a_km) { kk = (tid & 3) * 4; mm = (tid >> 2) + i * 64; } else { mm = (tid & 31) * 4; kk = (tid >> 5) + i * 8; }
+      const int64_t gm = m0 + mm, gk = k0 + kk;
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        int kk, cc;
-        if (g.b_km) { kk = tid & 15; cc = (tid >> 4) + i * 16; } else { cc = tid & 127; kk = (tid >> 7) + i * 2; }
-        int64_t gn;
-        if (gated) {
-          const int64_t ng = n0 + (cc >> 6) * 32 + (cc & 31);
-          gn = ng < N ? ((cc >> 5) & 1) * N + ng : b_rows;
+      for (int e = 0; e < 4; e++) f.a[i][e] = 0.f;
+      if (gm < M && gk < g.K) {
+        if (va) {
+          load4(g.a_km ? g.A + gm * g.lda + gk : g.A + gk * g.lda + gm, f.a[i]);
         } else {
-          gn = n0 + cc;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (g.a_km) { if (gk + e < g.K) f.a[i][e] = ldf(g.A, gm * g.lda + gk + e); }
+            else if (gm + e < M) f.a[i][e] = ldf(g.A, gk * g.lda + gm + e);
+          }
         }
-        const int64_t gk = k0 + kk;
-        float v = 0.f;
-        if (gn < b_rows && gk < g.K) v = g.b_km ? ldf(g.B, gn * g.ldb + gk) : ldf(g.B, gk * g.ldb + gn);
-        Bs[kk][cc] = v;
       }
-      __syncthreads();
-      // ---- 8 MFMA k-steps of 2: lane supplies A[row = lane % 32][k = lane / 32] and B[col = lane % 32][k = lane / 32]
-#pragma unroll
-      for (int kk = 0; kk < GBK; kk += 2) {
-        float a[2], bfrag[2];
-#pragma unroll
-        for (int i = 0; i < 2; i++) a[i] = As[kk + (lane >> 5)][wm * 64 + i * 32 + (lane & 31)];
-#pragma unroll
-        for (int j = 0; j < 2; j++) bfrag[j] = Bs[kk + (lane >> 5)][wn * 64 + j * 32 + (lane & 31)];
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-          for (int j = 0; j < 2; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bfrag[j], acc[i][j], 0, 0, 0);
-      }
-      __syncthreads();
     }
+    const bool vb = (reinterpret_cast<uintptr_t>(g.B) % (4 * sizeof(TI)) == 0) && (g.ldb & 3) == 0 &&
+                    (g.b_km ? (g.K & 3) == 0 : (N & 3) == 0);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      int kk, cc;
+      if (g.b_km) { kk = (tid & 3) * 4; cc = (tid >> 2) + i * 64; } else { cc = (tid & 31) * 4; kk = (tid >> 5) + i * 8; }
+      // global row of B for tile column cc (+ e along n when mn-major); b_rows = out of range
+      int64_t gn;
+      if (gated) {
+        const int64_t ng = n0 + (cc >> 6) * 32 + (cc & 31);
+        gn = ng < N ? ((cc >> 5) & 1) * N + ng : b_rows;
+      } else {
+        gn = n0 + cc < N ? n0 + cc : b_rows;
+      }
+      const int64_t gk = k0 + kk;
+#pragma unroll
+      for (int e = 0; e < 4; e++) f.b[i][e] = 0.f;
+      if (gn < b_rows && gk < g.K) {
+        if (vb) {
+          load4(g.b_km ? g.B + gn * g.ldb + gk : g.B + gk * g.ldb + gn, f.b[i]);
+        } else {
+          const int64_t n_left = (gated ? N - (n0 + (cc >> 6) * 32 + (cc & 31)) : N - (n0 + cc));
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (g.b_km) { if (gk + e < g.K) f.b[i][e] = ldf(g.B, gn * g.ldb + gk + e); }
+            else if (e < n_left) f.b[i][e] = ldf(g.B, gk * g.ldb + gn + e);
+          }
+        }
+      }
+    }
+  };
+  // f holds the step (seg, k0) points at: g is its segment
+  auto stash = [&](const Fetch& f, int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      if (g.a_km) {
+        const int kk = (tid & 3) * 4, mm = (tid >> 2) + i * 64;
+#pragma unroll
+        for (int e = 0; e < 4; e++) As[buf][kk + e][mm] = f.a[i][e];
+      } else {
+        const int mm = (tid & 31) * 4, kk = (tid >> 5) + i * 8;
+        *reinterpret_cast<float4*>(&As[buf][kk][mm]) = make_float4(f.a[i][0], f.a[i][1], f.a[i][2], f.a[i][3]);
+      }
+      if (g.b_km) {
+        const int kk = (tid & 3) * 4, cc = (tid >> 2) + i * 64;
+#pragma unroll
+        for (int e = 0; e < 4; e++) Bs[buf][kk + e][cc] = f.b[i][e];
+      } else {
+        const int cc = (tid & 31) * 4, kk = (tid >> 5) + i * 8;
+        *reinterpret_cast<float4*>(&Bs[buf][kk][cc]) = make_float4(f.b[i][0], f.b[i][1], f.b[i][2], f.b[i][3]);
+      }
+    }
+  };
+  // advance (seg, k0) to the next step; false at the end
+  auto advance = [&]() -> bool {
+    k0 += GBK;
+    if (k0 < g.K) return true;
+    if (++seg >= nseg) return false;
+    g = segment(seg);
+    k0 = 0;
+    return true;
+  };
+
+  Fetch f;
+  fetch(f);
+  stash(f, 0);
+  __syncthreads();
+  int buf = 0;
+  for (;;) {
+    const bool more = advance();
+    if (more) fetch(f);  // in flight while the matrix cores run
+#pragma unroll
+    for (int kk = 0; kk < GBK; kk += 2) {
+      float a[2], bfrag[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) a[i] = As[buf][kk + (lane >> 5)][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < 2; j++) bfrag[j] = Bs[buf][kk + (lane >> 5)][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bfrag[j], acc[i][j], 0, 0, 0);
+    }
+    if (!more) break;
+    stash(f, buf ^ 1);  // the other buffer: its last readers passed the previous barrier
+    __syncthreads();
+    buf ^= 1;
   }
 
   // ---- epilogue: accumulator register r of a 32 x 32 block is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
