@@ -1,11 +1,12 @@
-"""LeanFFN fwd+bwd throughput on one MI355X: BASELINE config 3 (hidden 4096, intermediate 16384, GeGLU, bf16 weights, fp32
+"""LeanFFN fwd+bwd throughput on one MI355X: benchmark config 3 (hidden 4096, intermediate 16384, GeGLU, bf16 weights, fp32
 residual stream, x [2, 2048, 4096]).  Prints one JSON line.
 
     python bench.py --gpus 1 --steps 20 --warmup 5
 
 A step is one forward + backward of the module on a resident synthetic batch (parameter gradients produced, no optimizer).
-`roofline` is computed from HIP events recorded around every launch of the tiled bf16 MFMA GEMM kernel during the timed
-steps; `cpu_baseline` times the CPU oracle (tests' checker, not the product) on a bounded sample of the same workload.
+K steps are timed by wall clock; the same K steps are then repeated with a HIP event pair around every kernel launch
+(recorded by the library on the launch stream) and `roofline` is computed from the GEMM launches of that pass;
+`cpu_baseline` times the CPU oracle (tests' checker, not the product) on a bounded sample of the same workload.
 """
 import argparse
 import json
@@ -21,7 +22,7 @@ PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk/CU x 2.4 GHz, dense
 PEAK_FP32_TFLOPS = 157.3   # fp32 matrix cores: the fp32 path computes there
 
 
-# BASELINE.json configurations that fit one GPU; the default (and the only one the metric is quoted on) is config 3
+# benchmark configurations that fit one GPU; the default (and the only one the metric is quoted on) is config 3
 CONFIGS = {
     "c1": dict(batch=8, seq=512, hidden=768, inter=3072, gated=True, std=0.02, dropout=0.0, dtype="fp32", sparse=False,
                name="config1: LeanFFN dense GeGLU fwd+bwd, hidden 768, intermediate 3072, x [8,512,768], fp32"),
@@ -106,7 +107,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing (profiling runs)")
-    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS), help="BASELINE.json configuration (default: the "
+    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS), help="benchmark configuration (default: the "
                     "headline config 3; the others are reported for reference)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -206,7 +207,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
-        sample = min(256, tokens)
+        sample = min(2048, tokens)  # about 10 s of host work with the warm-up
         value, sec = cpu_baseline(torch, 4096, 16384, 0.01, sample, iters=3)
         result["cpu_baseline"] = {
             "value": value, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",

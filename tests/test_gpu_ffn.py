@@ -199,7 +199,7 @@ def _c1():
 
 
 def test_config1_fp32_against_cpu_oracle():
-    """BASELINE config 1: fp32, hidden 768, intermediate 3072, GeGLU, eps 1e-5, x [8, 512, 768]; oracle on the host cores"""
+    """benchmark config 1: fp32, hidden 768, intermediate 3072, GeGLU, eps 1e-5, x [8, 512, 768]; oracle on the host cores"""
     ffn, x, dy = _c1()
     _compare(ffn.to(DEV), x, dy, torch.float32)
 
@@ -319,19 +319,19 @@ def _full_size_checks(ffn, x, dy, mask_p):
 
 
 def test_config2_bf16_full_size():
-    """BASELINE config 2: bf16, hidden 2048, intermediate 8192, plain GELU, dropout 0.1, x [4, 2048, 2048]"""
+    """benchmark config 2: bf16, hidden 2048, intermediate 8192, plain GELU, dropout 0.1, x [4, 2048, 2048]"""
     ffn, x, dy = _headline(2048, 8192, False, 0.02, 0.1, (4, 2048))
     _full_size_checks(ffn, x, dy, 0.1)
 
 
 def test_config3_bf16_full_size_headline():
-    """BASELINE config 3 (headline): bf16, hidden 4096, intermediate 16384, GeGLU, x [2, 2048, 4096], weights ~N(0, 0.01)"""
+    """benchmark config 3 (headline): bf16, hidden 4096, intermediate 16384, GeGLU, x [2, 2048, 4096], weights ~N(0, 0.01)"""
     ffn, x, dy = _headline(4096, 16384, True, 0.01, 0.0, (2, 2048))
     _full_size_checks(ffn, x, dy, 0.0)
 
 
 def test_config5_layer_shape_bf16_split_reduction():
-    """one FFN layer at BASELINE config 5's shape (hidden 768, intermediate 3072, GeGLU, 16 x 1024 tokens): the weight
+    """one FFN layer at benchmark config 5's shape (hidden 768, intermediate 3072, GeGLU, 16 x 1024 tokens): the weight
     gradients are [6144, 768] and [768, 3072], too few 256 x 256 tiles for 256 CUs, so their reduction over the tokens is
     split across workgroups and summed from fp32 partial results"""
     ffn, x, dy = _headline(768, 3072, True, 0.02, 0.0, (16, 1024))
@@ -340,7 +340,7 @@ def test_config5_layer_shape_bf16_split_reduction():
 
 @pytest.mark.parametrize("stretch", [True, False])
 def test_config4_pixelfly_bf16_full_size(stretch):
-    """BASELINE config 4: config 3's shape with PixelFly block-sparse projections (64 x 64 blocks, 7 of 64 blocks per block
+    """benchmark config 4: config 3's shape with PixelFly block-sparse projections (64 x 64 blocks, 7 of 64 blocks per block
     row: up-projection K/A = 7/56, down-projection 28/7) plus a rank-128 low-rank term, bf16"""
     g = torch.Generator().manual_seed(0)
     hidden, inter, rank = 4096, 16384, 128
