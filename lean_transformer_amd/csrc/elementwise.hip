@@ -285,6 +285,44 @@ __global__ void colreduce_kernel(int rows, int64_t stride, int cols, const float
   out[c] = s;
 }
 
+// same, 16 row lanes x 16 column lanes of 4 columns per workgroup: short dependent chains, 16-byte loads
+__global__ __launch_bounds__(256) void colreduce4_kernel(int rows, int64_t stride, int cols, const float* __restrict__ partial,
+                                                         float* __restrict__ out) {
+  __shared__ float red[16][16][5];
+  const int cl = threadIdx.x & 15, rl = threadIdx.x >> 4;
+  const int c = (blockIdx.x * 16 + cl) * 4;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < cols) {
+    for (int r = rl; r < rows; r += 16) {
+      float v[4];
+      load4(partial + (int64_t)r * stride + c, v);
+#pragma unroll
+      for (int e = 0; e < 4; e++) s[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) red[rl][cl][e] = s[e];
+  __syncthreads();
+  if (rl == 0 && c < cols) {
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      o[e] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 16; q++) o[e] += red[q][cl][e];
+    }
+    store4(out + c, o);
+  }
+}
+
+// out[c] = sum of `rows` rows of partial: picks the vector kernel when the layout allows
+static void launch_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream) {
+  if ((cols & 3) == 0 && (stride & 3) == 0 && lt_aligned(partial, 16) && lt_aligned(out, 16))
+    hipLaunchKernelGGL(colreduce4_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(256), 0, stream, rows, stride, cols, partial, out);
+  else
+    hipLaunchKernelGGL(colreduce_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, stream, rows, stride, cols, partial, out);
+}
+
 // partial[blockIdx.y][c] = sum over this row-slice of in[t, c]; 64 column lanes x 4 row lanes per workgroup
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_partial_kernel(int64_t rows, int cols, int64_t ld, const T* __restrict__ in,
@@ -318,6 +356,54 @@ __global__ __launch_bounds__(256) void colsum_partial8_kernel(int64_t rows, int 
       load8(in + r * ld + c, v);
 #pragma unroll
       for (int e = 0; e < 8; e++) s[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) red[rl][cl][e] = s[e];
+  __syncthreads();
+  if (rl == 0 && c < cols) {
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      o[e] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; q++) o[e] += red[q][cl][e];
+    }
+    store8(partial + (int64_t)blockIdx.y * cols + c, o);
+  }
+}
+
+// dropout replay + cast of a [rows, cols] gradient with the column sums of what it writes (the bias gradient of the layer
+// the result feeds), in the work decomposition of colsum_partial8_kernel
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void dropout_cast_colsum_kernel(int64_t rows, int cols, const TI* __restrict__ in,
+                                                                  TO* __restrict__ out, DropoutParams drop,
+                                                                  int64_t rows_per_slice, float* __restrict__ partial) {
+  __shared__ float red[8][32][9];
+  const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int c = (blockIdx.x * 32 + cl) * 8;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice, r1 = min(rows, r0 + rows_per_slice);
+  float s[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) s[e] = 0.f;
+  if (c < cols) {
+    for (int64_t r = r0 + rl; r < r1; r += 8) {
+      const int64_t idx = r * cols + c;
+      float v[8];
+      load8(in + idx, v);
+      if (drop.p > 0.f) {
+        bool k0[4], k1[4];
+        dropout_keep4(drop, idx, k0);
+        dropout_keep4(drop, idx + 4, k1);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          v[e] = k0[e] ? v[e] * drop.scale : 0.f;
+          v[4 + e] = k1[e] ? v[4 + e] * drop.scale : 0.f;
+        }
+      }
+      store8(out + idx, v);
+#pragma unroll
+      for (int e = 0; e < 8; e++) s[e] += (float)(TO)v[e];  // sums of the values as stored
     }
   }
 #pragma unroll
@@ -539,10 +625,10 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   }
   if (dweight) {
     // partial rows alternate (dweight, dbias): stride 2 * H between them
-    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, partial_rows, (int64_t)2 * H, H,
-                       partial, dweight);
-    hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(H, 256)), dim3(256), 0, stream, partial_rows, (int64_t)2 * H, H,
-                       partial + H, dbias);
+    launch_colreduce(partial_rows, (int64_t)2 * H, H,
+                       partial, dweight, stream);
+    launch_colreduce(partial_rows, (int64_t)2 * H, H,
+                       partial + H, dbias, stream);
     LT_LAUNCH_CHECK();
   }
   return LT_OK;
@@ -577,8 +663,7 @@ int lt_colsum(int64_t rows, int cols, int64_t ld, int dtype, const void* in, flo
     else
       hipLaunchKernelGGL((colsum_partial_kernel<bf16>), grid, block, 0, stream, rows, cols, ld, (const bf16*)in, rps, partial);
   }
-  hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(cols, 256)), dim3(256), 0, stream, slices, (int64_t)cols, cols,
-                     partial, out);
+  launch_colreduce(slices, (int64_t)cols, cols, partial, out, stream);
   LT_LAUNCH_CHECK();
   return LT_OK;
 }
@@ -626,6 +711,35 @@ int lt_dropout_cast(int64_t n, int in_dtype, const void* in, int out_dtype, void
   return LT_OK;
 }
 
+// lt_dropout_cast of a [rows, cols] tensor plus colsum[c] = sum over rows of the result; workspace as for lt_colsum
+int lt_dropout_cast_colsum(int64_t rows, int cols, int in_dtype, const void* in, int out_dtype, void* out,
+                           const DropoutParams& drop, float* colsum, void* workspace, size_t workspace_bytes,
+                           hipStream_t stream) {
+  LT_REQUIRE(rows > 0 && cols > 0 && in && out && colsum, LT_ERR_BAD_ARG, "dropout + column sums: bad arguments");
+  LT_REQUIRE(workspace && workspace_bytes >= lt_colsum_workspace(rows, cols), LT_ERR_WORKSPACE,
+             "dropout + column sums: workspace of %zu bytes needed", lt_colsum_workspace(rows, cols));
+  if ((cols & 7) != 0 || !lt_aligned(in, 16) || !lt_aligned(out, 16) || !lt_aligned(workspace, 16)) {
+    LT_TRY(lt_dropout_cast(rows * cols, in_dtype, in, out_dtype, out, drop, stream));
+    return lt_colsum(rows, cols, cols, out_dtype, out, colsum, workspace, workspace_bytes, stream);
+  }
+  LtProfileScope scope("dropout_replay_cast", 0.0, (double)rows * cols * (lt_dtype_size(in_dtype) + lt_dtype_size(out_dtype)),
+                       stream);
+  const int slices = colsum_slices(rows);
+  const int64_t rps = (rows + slices - 1) / slices;
+  float* partial = (float*)workspace;
+  dim3 grid(blocks_for(cols, 256), slices), block(256);
+  const int key = (in_dtype == LT_BF16) * 2 + (out_dtype == LT_BF16);
+  switch (key) {
+    case 0: hipLaunchKernelGGL((dropout_cast_colsum_kernel<float, float>), grid, block, 0, stream, rows, cols, (const float*)in, (float*)out, drop, rps, partial); break;
+    case 1: hipLaunchKernelGGL((dropout_cast_colsum_kernel<float, bf16>), grid, block, 0, stream, rows, cols, (const float*)in, (bf16*)out, drop, rps, partial); break;
+    case 2: hipLaunchKernelGGL((dropout_cast_colsum_kernel<bf16, float>), grid, block, 0, stream, rows, cols, (const bf16*)in, (float*)out, drop, rps, partial); break;
+    default: hipLaunchKernelGGL((dropout_cast_colsum_kernel<bf16, bf16>), grid, block, 0, stream, rows, cols, (const bf16*)in, (bf16*)out, drop, rps, partial); break;
+  }
+  launch_colreduce(slices, (int64_t)cols, cols, partial, colsum, stream);
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
 int lt_dropout_mask_launch(int64_t n, uint8_t* keep, const DropoutParams& drop, hipStream_t stream) {
   LT_REQUIRE(n > 0 && keep, LT_ERR_BAD_ARG, "dropout mask: bad arguments");
   hipLaunchKernelGGL(dropout_mask_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, n, keep, drop);
@@ -650,7 +764,7 @@ int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t c
 int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream) {
   LT_REQUIRE(rows > 0 && cols > 0 && partial && out, LT_ERR_BAD_ARG, "colreduce: bad arguments");
   LtProfileScope scope("colreduce", 0.0, (double)cols * 4.0 * (rows + 1), stream);
-  hipLaunchKernelGGL(colreduce_kernel, dim3(blocks_for(cols, 256)), dim3(256), 0, stream, rows, stride, cols, partial, out);
+  launch_colreduce(rows, stride, cols, partial, out, stream);
   LT_LAUNCH_CHECK();
   return LT_OK;
 }

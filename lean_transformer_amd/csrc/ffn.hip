@@ -383,8 +383,14 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
 
   // gradient entering the down-projection: dropout replayed on dy, then (optionally) back through the post-LN
   const void* g = s.g;
+  lt_linear_grads h2o_grads = grads->h2o;
   if (d.dropout_p == 0.f && io == cdt) {
     g = dy;
+  } else if (h2o_grads.bias && !d.post_ln_weight) {
+    // the same pass also sums the columns of g: the down-projection's bias gradient
+    LT_TRY(lt_dropout_cast_colsum(T, (int)H, io, dy, cdt, s.g, drop, (float*)h2o_grads.bias, s.h2o.colsum, s.h2o.colsum_bytes,
+                                  stream));
+    h2o_grads.bias = nullptr;
   } else {
     LT_TRY(lt_dropout_cast(T * H, io, dy, cdt, s.g, drop, stream));
   }
@@ -403,7 +409,7 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
     memset(&e, 0, sizeof(e));
     e.pre = saved->pre_activation; e.ld_pre = N1; e.dpre = s.dpre; e.hid = s.hid; e.ld_hid = I;
     e.gated = d.gated; e.act = d.act; e.inter = I;
-    LT_TRY(linear_backward_impl(d.h2o, T, cdt, s.hid, g, saved->h2o_lowrank_hid, EPI_ACT_BWD, e, grads->h2o, s.h2o, io,
+    LT_TRY(linear_backward_impl(d.h2o, T, cdt, s.hid, g, saved->h2o_lowrank_hid, EPI_ACT_BWD, e, h2o_grads, s.h2o, io,
                                 stream, grads->i2h.bias ? s.act_colsum : nullptr, &bias_from_epilogue));
   }
   lt_linear_grads i2h_grads = grads->i2h;

@@ -16,6 +16,9 @@ int lt_colsum(int64_t rows, int cols, int64_t ld, int dtype, const void* in, flo
 int lt_act_forward(int64_t T, int64_t I, int gated, int act, int dtype, const void* pre, void* hid, hipStream_t stream);
 int lt_act_backward(int64_t T, int64_t I, int gated, int act, int dtype, const void* pre, const void* dhid, void* dpre,
                     hipStream_t stream);
+int lt_dropout_cast_colsum(int64_t rows, int cols, int in_dtype, const void* in, int out_dtype, void* out,
+                           const DropoutParams& drop, float* colsum, void* workspace, size_t workspace_bytes,
+                           hipStream_t stream);
 int lt_dropout_cast(int64_t n, int in_dtype, const void* in, int out_dtype, void* out, const DropoutParams& drop,
                     hipStream_t stream);
 int lt_dropout_mask_launch(int64_t n, uint8_t* keep, const DropoutParams& drop, hipStream_t stream);
