@@ -796,13 +796,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   float colsum[16];  // EPI_ACT_BWD: column sums of this lane's 8 (+ 8) dpre columns over the rows it writes
 #pragma unroll
   for (int e = 0; e < 16; e++) colsum[e] = 0.f;
-#pragma unroll
-  for (int i = 0; i < FM; i++) {
+  // accumulators of strip I -> this wavefront's staging buffer
+  auto stage_strip = [&](auto I) {
+    constexpr int i = decltype(I)::value;
 #pragma unroll
     for (int j = 0; j < FN; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) *staged(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), j * 32 + (lane & 31)) = acc[i][j][r];
     __builtin_amdgcn_wave_barrier();
+  };
+  auto for_each_strip = [&](auto&& strip) {
+    static_assert(FM == 4, "four 32-row strips per wavefront");
+    strip(std::integral_constant<int, 0>{});
+    strip(std::integral_constant<int, 1>{});
+    strip(std::integral_constant<int, 2>{});
+    strip(std::integral_constant<int, 3>{});
+  };
+  auto generic_strip = [&](auto I) {
+    constexpr int i = decltype(I)::value;
+    stage_strip(I);
     const int64_t mrow0 = m0 + wm * WTM + i * 32;
     if (pair) {
       // columns [0, WTN/2) of the sub-tile are gate columns, [WTN/2, WTN) the matching linear columns
@@ -848,6 +860,93 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       }
     }
     __builtin_amdgcn_wave_barrier();
+  };
+  // EPI_ACT_BWD, the usual case (whole tile in range, tanh GELU, h wanted): straight-line strips.  The pre-activation reads
+  // of ACT_WINDOW rows are in flight at any time -- the first window goes out before the strip is staged -- and, with no
+  // branches in between, each row waits only for its own reads.
+  constexpr int ACT_WINDOW = 3;
+  auto act_bwd_strip = [&](auto I, auto G) {
+    constexpr int i = decltype(I)::value;
+    constexpr bool GATED = decltype(G)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * WTN + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    EpiLoad win[ACT_WINDOW];
+#pragma unroll
+    for (int it = 0; it < ACT_WINDOW; it++) win[it] = epi_load_pre8<GATED>(epi, mlane + it * ROWS_PER_IT, n);
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
+      float v[8];
+      const float* sv = staged(row, c);
+#pragma unroll
+      for (int e = 0; e < 8; e++) v[e] = sv[e];
+      epi_act_bwd8_gelu<GATED>(epi, mlane + it * ROWS_PER_IT, n, v, win[it % ACT_WINDOW], colsum);
+      if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_pre8<GATED>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  // EPI_STORE and EPI_OUT, same idea: whole tile in range, no dropout, residual and bias present.  (EPI_ACT_FWD reads nothing
+  // and a straight-line variant of it overflows the register budget of the main loop: it keeps the general strip.)
+  const bool whole_tile = m0 + BM <= p.M;
+  auto store_strip = [&](auto I, auto out_type) {
+    using TO = decltype(out_type);
+    constexpr int i = decltype(I)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * WTN + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      float v[8];
+      const float* sv = staged(it * ROWS_PER_IT + lane / LANES_PER_ROW, c);
+#pragma unroll
+      for (int e = 0; e < 8; e++) v[e] = sv[e];
+      epi_store8_plain<TO>(epi, mlane + it * ROWS_PER_IT, n, v);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto out_strip = [&](auto I, const float (&b)[8]) {
+    constexpr int i = decltype(I)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * WTN + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    EpiLoad win[ACT_WINDOW];
+#pragma unroll
+    for (int it = 0; it < ACT_WINDOW; it++) win[it] = epi_load_x8<TX>(epi, mlane + it * ROWS_PER_IT, n);
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      float v[8];
+      const float* sv = staged(it * ROWS_PER_IT + lane / LANES_PER_ROW, c);
+#pragma unroll
+      for (int e = 0; e < 8; e++) v[e] = sv[e];
+      epi_out8_residual<TX>(epi, mlane + it * ROWS_PER_IT, n, v, b, win[it % ACT_WINDOW]);
+      if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_x8<TX>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  if constexpr (KIND == EPI_ACT_BWD) {
+    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED && epi.hid != nullptr;
+    if (straight && epi.gated) for_each_strip([&](auto I) { act_bwd_strip(I, std::true_type{}); });
+    else if (straight) for_each_strip([&](auto I) { act_bwd_strip(I, std::false_type{}); });
+    else for_each_strip(generic_strip);
+  } else if constexpr (KIND == EPI_STORE) {
+    if (whole_tile && !epi.bias && epi.out_dtype == LT_F32) for_each_strip([&](auto I) { store_strip(I, float{}); });
+    else if (whole_tile && !epi.bias) for_each_strip([&](auto I) { store_strip(I, bf16{}); });
+    else for_each_strip(generic_strip);
+  } else {
+    if (whole_tile && epi.bias && epi.x && epi.drop.p == 0.f) {
+      float b[8];
+      load8(epi.bias + n0 + wn * WTN + (lane % (WTN / 8)) * 8, b);
+      for_each_strip([&](auto I) { out_strip(I, b); });
+    } else {
+      for_each_strip(generic_strip);
+    }
   }
   if constexpr (KIND == EPI_ACT_BWD) {
     if (epi.colsum) {

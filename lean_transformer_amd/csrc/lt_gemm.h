@@ -304,6 +304,85 @@ __device__ __forceinline__ void epi_act_bwd8_loaded(const EpiParams& e, int64_t 
   if (e.hid) store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, a);
 }
 
+// Straight-line epilogue bodies for the usual cases (whole tile in range, bias present, no dropout): the run-time choices of
+// the general functions above are made once per tile by the caller, not once per row; bias values of a lane's 8 columns
+// are loaded once per tile and passed in.
+template <typename TO> __device__ __forceinline__ void epi_store8_plain(const EpiParams& e, int64_t m, int64_t n, const float (&v)[8]) {
+  store8(reinterpret_cast<TO*>(e.out) + m * e.ldo + n, v);
+}
+
+// y = acc + bias + x, residual read ahead (no dropout)
+template <typename TX> __device__ __forceinline__ EpiLoad epi_load_x8(const EpiParams& e, int64_t m, int64_t n) {
+  EpiLoad l;
+  const TX* x = reinterpret_cast<const TX*>(e.x) + m * e.ldy + n;
+  l.a = *reinterpret_cast<const lt_u32x4*>(x);
+  if constexpr (sizeof(TX) == 4) l.b = *reinterpret_cast<const lt_u32x4*>(x + 4);
+  else l.b = l.a;
+  return l;
+}
+
+template <typename TX>
+__device__ __forceinline__ void epi_out8_residual(const EpiParams& e, int64_t m, int64_t n, float (&v)[8], const float (&b)[8],
+                                                  const EpiLoad& l) {
+  float r[8];
+  if constexpr (sizeof(TX) == 4) {
+    union { lt_u32x4 u[2]; float f[8]; } t;
+    t.u[0] = l.a;
+    t.u[1] = l.b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r[i] = t.f[i];
+  } else {
+    unpack_bf16x8(l.a, r);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] += b[i] + r[i];
+  store8(reinterpret_cast<TX*>(e.y) + m * e.ldy + n, v);
+}
+
+// EPI_ACT_BWD without run-time choices -- tanh-approximated GELU, gating fixed at compile time, h always written, rows known to
+// be in range: straight-line code, so the compiler can count exactly which of the reads in flight a row waits for
+template <bool GATED> __device__ __forceinline__ EpiLoad epi_load_pre8(const EpiParams& e, int64_t m, int64_t n) {
+  EpiLoad l;
+  const bf16* pre = reinterpret_cast<const bf16*>(e.pre) + m * e.ld_pre + n;
+  l.a = *reinterpret_cast<const lt_u32x4*>(pre);
+  if constexpr (GATED) l.b = *reinterpret_cast<const lt_u32x4*>(pre + e.inter);
+  else l.b = l.a;
+  return l;
+}
+
+template <bool GATED>
+__device__ __forceinline__ void epi_act_bwd8_gelu(const EpiParams& e, int64_t m, int64_t n, const float (&dh)[8],
+                                                  const EpiLoad& l, float (&cs)[16]) {
+  bf16* dpre = reinterpret_cast<bf16*>(e.dpre) + m * e.ld_pre + n;
+  float pg[8], a[8], da[8], o[8];
+  unpack_bf16x8(l.a, pg);
+#pragma unroll
+  for (int i = 0; i < 8; i++) act_eval<false>(LT_ACT_GELU_FUSED, pg[i], a[i], da[i]);
+  if constexpr (GATED) {
+    float pl[8];
+    unpack_bf16x8(l.b, pl);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * pl[i] * da[i];
+    store8(dpre, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) cs[i] += (float)(bf16)o[i];
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * a[i];
+    store8(dpre + e.inter, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) cs[8 + i] += (float)(bf16)o[i];
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] *= pl[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[i] = dh[i] * da[i];
+    store8(dpre, o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) cs[i] += (float)(bf16)o[i];
+  }
+  store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, a);
+}
+
 template <typename TX>
 __device__ __forceinline__ void epi_out8_loaded(const EpiParams& e, int64_t m, int64_t n, float (&v)[8], const EpiLoad& l) {
   add_bias8(e.bias, n, v);
