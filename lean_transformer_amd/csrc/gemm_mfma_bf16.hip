@@ -540,13 +540,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   const int64_t m0 = (int64_t)tm * BM;
   const int64_t n0 = (int64_t)tn * (gated ? BN / 2 : BN);
 
+  // The accumulators start at the bias of their column (a lane holds one column per 32-wide block), so no epilogue has to
+  // add it.  Gated forward: blocks 0, 1 of a wavefront are gate columns, 2, 3 the matching linear columns.
+  float bias0[FN];
+#pragma unroll
+  for (int j = 0; j < FN; j++) {
+    bias0[j] = 0.f;
+    if (p.epi.bias) {
+      const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) + n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31)
+                                : n0 + wn * WTN + j * 32 + (lane & 31);
+      bias0[j] = p.epi.bias[col];
+    }
+  }
   f32x16 acc[FM][FN];
 #pragma unroll
   for (int i = 0; i < FM; i++)
 #pragma unroll
     for (int j = 0; j < FN; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; r++) acc[i][j][r] = bias0[j];
 
   const int kt_all = (int)((p.K[0] + DK - 1) / DK) + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
   // split-k (one k-segment only): this workgroup walks k-steps [kt_begin, kt_begin + kt_total) of kt_all; the slices are
@@ -785,6 +797,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   //      Staged column c of row r sits at c ^ 32 when bit 2 of r is set: the two half-waves of a transposing write (rows
   //      r and r + 4, same columns) then hit different banks without padding the rows.
   EpiParams epi = p.epi;
+  epi.bias = nullptr;  // already in the accumulators
   if (KIND == EPI_STORE && p.ksplit > 1) epi.out = reinterpret_cast<float*>(epi.out) + (int64_t)blockIdx.y * p.split_stride;
   float* stage = reinterpret_cast<float*>(wave == 0   ? (A_KM ? a_d0 : a_s0)
                                           : wave == 1 ? (A_KM ? a_d1 : a_s1)
@@ -888,9 +901,31 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     }
     __builtin_amdgcn_wave_barrier();
   };
-  // EPI_STORE and EPI_OUT, same idea: whole tile in range, no dropout, residual and bias present.  (EPI_ACT_FWD reads nothing
-  // and a straight-line variant of it overflows the register budget of the main loop: it keeps the general strip.)
+  // The other kinds, same idea: whole tile in range, tanh GELU, no dropout, residual present.
   const bool whole_tile = m0 + BM <= p.M;
+  auto act_fwd_strip = [&](auto I, auto G) {
+    constexpr int i = decltype(I)::value;
+    constexpr bool GATED = decltype(G)::value;
+    constexpr int LANES_PER_ROW = (GATED ? WTN / 2 : WTN) / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * (GATED ? WTN / 2 : WTN) + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
+      float v0[8], v1[8];
+      const float* s0 = staged(row, c);
+      const float* s1 = staged(row, GATED ? WTN / 2 + c : c);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        v0[e] = s0[e];
+        v1[e] = s1[e];
+      }
+      epi_act_fwd8_gelu<GATED>(epi, mlane + it * ROWS_PER_IT, n, v0, v1);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
   auto store_strip = [&](auto I, auto out_type) {
     using TO = decltype(out_type);
     constexpr int i = decltype(I)::value;
@@ -909,7 +944,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     }
     __builtin_amdgcn_wave_barrier();
   };
-  auto out_strip = [&](auto I, const float (&b)[8]) {
+  auto out_strip = [&](auto I) {
     constexpr int i = decltype(I)::value;
     constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
     const int c = (lane % LANES_PER_ROW) * 8;
@@ -925,7 +960,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       const float* sv = staged(it * ROWS_PER_IT + lane / LANES_PER_ROW, c);
 #pragma unroll
       for (int e = 0; e < 8; e++) v[e] = sv[e];
-      epi_out8_residual<TX>(epi, mlane + it * ROWS_PER_IT, n, v, b, win[it % ACT_WINDOW]);
+      epi_out8_residual<TX>(epi, mlane + it * ROWS_PER_IT, n, v, win[it % ACT_WINDOW]);
       if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_x8<TX>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
     }
     __builtin_amdgcn_wave_barrier();
@@ -935,15 +970,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     if (straight && epi.gated) for_each_strip([&](auto I) { act_bwd_strip(I, std::true_type{}); });
     else if (straight) for_each_strip([&](auto I) { act_bwd_strip(I, std::false_type{}); });
     else for_each_strip(generic_strip);
+  } else if constexpr (KIND == EPI_ACT_FWD) {
+    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED;
+    if (straight && pair) for_each_strip([&](auto I) { act_fwd_strip(I, std::true_type{}); });
+    else if (straight) for_each_strip([&](auto I) { act_fwd_strip(I, std::false_type{}); });
+    else for_each_strip(generic_strip);
   } else if constexpr (KIND == EPI_STORE) {
-    if (whole_tile && !epi.bias && epi.out_dtype == LT_F32) for_each_strip([&](auto I) { store_strip(I, float{}); });
-    else if (whole_tile && !epi.bias) for_each_strip([&](auto I) { store_strip(I, bf16{}); });
+    if (whole_tile && epi.out_dtype == LT_F32) for_each_strip([&](auto I) { store_strip(I, float{}); });
+    else if (whole_tile) for_each_strip([&](auto I) { store_strip(I, bf16{}); });
     else for_each_strip(generic_strip);
   } else {
-    if (whole_tile && epi.bias && epi.x && epi.drop.p == 0.f) {
-      float b[8];
-      load8(epi.bias + n0 + wn * WTN + (lane % (WTN / 8)) * 8, b);
-      for_each_strip([&](auto I) { out_strip(I, b); });
+    if (whole_tile && epi.x && epi.drop.p == 0.f) {
+      for_each_strip(out_strip);
     } else {
       for_each_strip(generic_strip);
     }

@@ -307,11 +307,30 @@ __device__ __forceinline__ void epi_act_bwd8_loaded(const EpiParams& e, int64_t 
 // Straight-line epilogue bodies for the usual cases (whole tile in range, bias present, no dropout): the run-time choices of
 // the general functions above are made once per tile by the caller, not once per row; bias values of a lane's 8 columns
 // are loaded once per tile and passed in.
+// forward activation with the tanh GELU fixed (bias already in the accumulators)
+template <bool GATED>
+__device__ __forceinline__ void epi_act_fwd8_gelu(const EpiParams& e, int64_t m, int64_t n, float (&vg)[8], float (&vl)[8]) {
+  float h[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    vg[i] = to_f32((bf16)vg[i]);  // the activation sees the stored (rounded) pre-activation, as backward will
+    h[i] = act_value<false>(LT_ACT_GELU_FUSED, vg[i]);
+    if constexpr (GATED) {
+      vl[i] = to_f32((bf16)vl[i]);
+      h[i] *= vl[i];
+    }
+  }
+  bf16* pre = reinterpret_cast<bf16*>(e.pre) + m * e.ld_pre + n;
+  store8(pre, vg);
+  if constexpr (GATED) store8(pre + e.inter, vl);
+  store8(reinterpret_cast<bf16*>(e.hid) + m * e.ld_hid + n, h);
+}
+
 template <typename TO> __device__ __forceinline__ void epi_store8_plain(const EpiParams& e, int64_t m, int64_t n, const float (&v)[8]) {
   store8(reinterpret_cast<TO*>(e.out) + m * e.ldo + n, v);
 }
 
-// y = acc + bias + x, residual read ahead (no dropout)
+// y = acc + x, residual read ahead (no dropout; the bias is in the accumulators already)
 template <typename TX> __device__ __forceinline__ EpiLoad epi_load_x8(const EpiParams& e, int64_t m, int64_t n) {
   EpiLoad l;
   const TX* x = reinterpret_cast<const TX*>(e.x) + m * e.ldy + n;
@@ -322,8 +341,7 @@ template <typename TX> __device__ __forceinline__ EpiLoad epi_load_x8(const EpiP
 }
 
 template <typename TX>
-__device__ __forceinline__ void epi_out8_residual(const EpiParams& e, int64_t m, int64_t n, float (&v)[8], const float (&b)[8],
-                                                  const EpiLoad& l) {
+__device__ __forceinline__ void epi_out8_residual(const EpiParams& e, int64_t m, int64_t n, float (&v)[8], const EpiLoad& l) {
   float r[8];
   if constexpr (sizeof(TX) == 4) {
     union { lt_u32x4 u[2]; float f[8]; } t;
@@ -335,7 +353,7 @@ __device__ __forceinline__ void epi_out8_residual(const EpiParams& e, int64_t m,
     unpack_bf16x8(l.a, r);
   }
 #pragma unroll
-  for (int i = 0; i < 8; i++) v[i] += b[i] + r[i];
+  for (int i = 0; i < 8; i++) v[i] += r[i];
   store8(reinterpret_cast<TX*>(e.y) + m * e.ldy + n, v);
 }
 
