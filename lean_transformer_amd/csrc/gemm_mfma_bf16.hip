@@ -54,6 +54,14 @@ template <int READS, int MFMAS, int G = 0> struct SchedInterleave {
 // groups: output blocks (FWD, tile 256 x 64), input blocks (DX, tile 256 x 64), or (input block, four of its active
 // output blocks) (DW, tile 256 x 64: four gathered dY column blocks against one X column block, reduced over tokens;
 // the four weight-gradient blocks are adjacent in the native [in_blocks, A, 64, 64] order).
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
+template <typename F, int... Is> __device__ __forceinline__ void lt_static_for_impl(F& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void lt_static_for(F&& f) {
+  lt_static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX, int SP = SPARSE_NONE>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int NT = WM * WN * 64;
@@ -299,14 +307,33 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     n_base = 0;
     m_base = 0;
   }
+  // The bias is added while the accumulators are staged (a lane holds one column per 32-wide block), so no epilogue body has
+  // to.  Gated forward: the first half of a wavefront's column blocks are gate columns, the second half the matching linear
+  // columns.  (A split reduction passes no bias; the sparse weight-gradient walk has none.)
+  float bias0[FN];
 #pragma unroll
-  for (int i = 0; i < FM; i++) {
+  for (int j = 0; j < FN; j++) {
+    bias0[j] = 0.f;
+    if (SP != SPARSE_DW && epi.bias) {
+      const int64_t col = gated ? (j >= FN / 2 ? epi.inter : 0) + n0 + wn * (WTN / 2) + (j % (FN / 2 > 0 ? FN / 2 : 1)) * 32 + (lane & 31)
+                                : n0 + wn * WTN + j * 32 + (lane & 31);
+      bias0[j] = epi.bias[col];
+    }
+  }
+  epi.bias = nullptr;
+  auto stage_strip = [&](auto I) __attribute__((always_inline)) {
+    constexpr int i = decltype(I)::value;
 #pragma unroll
     for (int j = 0; j < FN; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++)
-        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * STAGE_LD + j * 32 + (lane & 31)] = acc[i][j][r];
+        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * STAGE_LD + j * 32 + (lane & 31)] = acc[i][j][r] + bias0[j];
     __builtin_amdgcn_wave_barrier();
+  };
+  // general strip: every choice (row in range, output type, activation, dropout, ...) is made per row
+  auto generic_strip = [&](auto I) __attribute__((always_inline)) {
+    constexpr int i = decltype(I)::value;
+    stage_strip(I);
     const int64_t mrow0 = m_base + wm * WTM + i * 32;
     if (pair) {
       // columns [0, WTN/2) of the sub-tile are gate columns, [WTN/2, WTN) the matching linear columns
@@ -320,7 +347,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
           vg[e] = stage[row * STAGE_LD + c + e];
           vl[e] = stage[row * STAGE_LD + WTN / 2 + c + e];
         }
-        if (m < p.M) epi_act_fwd_gated8(p.epi, m, n0 + wn * (WTN / 2) + c, vg, vl);
+        if (m < p.M) epi_act_fwd_gated8(epi, m, n0 + wn * (WTN / 2) + c, vg, vl);
       }
     } else {
       constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW;
@@ -340,6 +367,75 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       }
     }
     __builtin_amdgcn_wave_barrier();
+  };
+  // Straight-line strips for whole tiles in the usual configurations: the choices are made once per tile and the global
+  // reads of a strip (pre-activations, residual) go out before the strip is staged.
+  constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+  const int lane_c = (lane % LANES_PER_ROW) * 8;
+  const int64_t lane_n = n_base + lane_c;
+  auto lane_row = [&](int i) -> int64_t { return m_base + wm * WTM + i * 32 + lane / LANES_PER_ROW; };
+  auto read_staged = [&](int it, float (&v)[8]) {
+    const float* sv = &stage[(it * ROWS_PER_IT + lane / LANES_PER_ROW) * STAGE_LD + lane_c];
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = sv[e];
+  };
+  auto store_strip = [&](auto I, auto out_type) __attribute__((always_inline)) {
+    using TO = decltype(out_type);
+    constexpr int i = decltype(I)::value;
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      float v[8];
+      read_staged(it, v);
+      epi_store8_plain<TO>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n, v);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto act_bwd_strip = [&](auto I, auto G) __attribute__((always_inline)) {
+    constexpr int i = decltype(I)::value;
+    constexpr bool GATED = decltype(G)::value;
+    float unused[16];
+    EpiLoad rows[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) rows[it] = epi_load_pre8<GATED>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n);
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      float v[8];
+      read_staged(it, v);
+      epi_act_bwd8_gelu<GATED>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n, v, rows[it], unused);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto out_strip = [&](auto I) __attribute__((always_inline)) {
+    constexpr int i = decltype(I)::value;
+    EpiLoad rows[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) rows[it] = epi_load_x8<TX>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n);
+    stage_strip(I);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      float v[8];
+      read_staged(it, v);
+      epi_out8_residual<TX>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n, v, rows[it]);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  const bool whole_tile = m_base + BM <= m_limit;
+  if constexpr (NIT <= 4 && KIND == EPI_STORE) {
+    if (whole_tile && epi.out_dtype == LT_F32) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { store_strip(I, float{}); });
+    else if (whole_tile) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { store_strip(I, bf16{}); });
+    else lt_static_for<FM>(generic_strip);
+  } else if constexpr (NIT <= 4 && KIND == EPI_ACT_BWD) {
+    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED && epi.hid != nullptr;
+    if (straight && epi.gated) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { act_bwd_strip(I, std::true_type{}); });
+    else if (straight) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { act_bwd_strip(I, std::false_type{}); });
+    else lt_static_for<FM>(generic_strip);
+  } else if constexpr (NIT <= 4 && KIND == EPI_OUT) {
+    if (whole_tile && epi.x && epi.drop.p == 0.f) lt_static_for<FM>(out_strip);
+    else lt_static_for<FM>(generic_strip);
+  } else {
+    lt_static_for<FM>(generic_strip);
   }
 }
 
