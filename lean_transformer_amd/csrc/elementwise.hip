@@ -436,6 +436,56 @@ __global__ void act_fwd_kernel(int64_t T, int64_t I, int gated, int act, const T
   stf(hid, idx, a);
 }
 
+// 8 consecutive features per thread (16-byte accesses for bf16); I % 8 == 0 and 16-byte aligned rows
+template <typename TC>
+__global__ void act_fwd8_kernel(int64_t T, int64_t I, int gated, int act, const TC* __restrict__ pre, TC* __restrict__ hid) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (idx >= T * I) return;
+  const int64_t t = idx / I, i = idx % I;
+  const int64_t ldp = gated ? 2 * I : I;
+  float g[8], h[8];
+  load8(pre + t * ldp + i, g);
+#pragma unroll
+  for (int e = 0; e < 8; e++) h[e] = act_value<PRECISE>(act, g[e]);
+  if (gated) {
+    float l[8];
+    load8(pre + t * ldp + I + i, l);
+#pragma unroll
+    for (int e = 0; e < 8; e++) h[e] *= l[e];
+  }
+  store8(hid + idx, h);
+}
+
+template <typename TC>
+__global__ void act_bwd8_kernel(int64_t T, int64_t I, int gated, int act, const TC* __restrict__ pre,
+                                const TC* __restrict__ dhid, TC* __restrict__ dpre) {
+  constexpr bool PRECISE = sizeof(TC) == 4;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (idx >= T * I) return;
+  const int64_t t = idx / I, i = idx % I;
+  const int64_t ldp = gated ? 2 * I : I;
+  float g[8], a[8], da[8], dh[8], o[8];
+  load8(pre + t * ldp + i, g);
+  load8(dhid + idx, dh);
+#pragma unroll
+  for (int e = 0; e < 8; e++) act_eval<PRECISE>(act, g[e], a[e], da[e]);
+  if (gated) {
+    float l[8];
+    load8(pre + t * ldp + I + i, l);
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = dh[e] * l[e] * da[e];
+    store8(dpre + t * ldp + i, o);
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = dh[e] * a[e];
+    store8(dpre + t * ldp + I + i, o);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = dh[e] * da[e];
+    store8(dpre + t * ldp + i, o);
+  }
+}
+
 template <typename TC>
 __global__ void act_bwd_kernel(int64_t T, int64_t I, int gated, int act, const TC* __restrict__ pre,
                                const TC* __restrict__ dhid, TC* __restrict__ dpre) {
@@ -672,7 +722,13 @@ int lt_act_forward(int64_t T, int64_t I, int gated, int act, int dtype, const vo
   LT_REQUIRE(T > 0 && I > 0 && pre && hid, LT_ERR_BAD_ARG, "activation: bad arguments");
   LtProfileScope scope("activation_fwd", 0.0, (double)T * I * lt_dtype_size(dtype) * (gated ? 3 : 2), stream);
   dim3 grid(blocks_for(T * I, 256)), block(256);
-  if (dtype == LT_F32)
+  const bool vec = (I & 7) == 0 && lt_aligned(pre, 16) && lt_aligned(hid, 16);
+  if (vec) grid = dim3(blocks_for(T * I / 8, 256));
+  if (dtype == LT_F32 && vec)
+    hipLaunchKernelGGL((act_fwd8_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre, (float*)hid);
+  else if (vec)
+    hipLaunchKernelGGL((act_fwd8_kernel<bf16>), grid, block, 0, stream, T, I, gated, act, (const bf16*)pre, (bf16*)hid);
+  else if (dtype == LT_F32)
     hipLaunchKernelGGL((act_fwd_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre, (float*)hid);
   else
     hipLaunchKernelGGL((act_fwd_kernel<bf16>), grid, block, 0, stream, T, I, gated, act, (const bf16*)pre, (bf16*)hid);
@@ -685,7 +741,15 @@ int lt_act_backward(int64_t T, int64_t I, int gated, int act, int dtype, const v
   LT_REQUIRE(T > 0 && I > 0 && pre && dhid && dpre, LT_ERR_BAD_ARG, "activation backward: bad arguments");
   LtProfileScope scope("activation_bwd", 0.0, (double)T * I * lt_dtype_size(dtype) * (gated ? 5 : 3), stream);
   dim3 grid(blocks_for(T * I, 256)), block(256);
-  if (dtype == LT_F32)
+  const bool vec = (I & 7) == 0 && lt_aligned(pre, 16) && lt_aligned(dhid, 16) && lt_aligned(dpre, 16);
+  if (vec) grid = dim3(blocks_for(T * I / 8, 256));
+  if (dtype == LT_F32 && vec)
+    hipLaunchKernelGGL((act_bwd8_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre,
+                       (const float*)dhid, (float*)dpre);
+  else if (vec)
+    hipLaunchKernelGGL((act_bwd8_kernel<bf16>), grid, block, 0, stream, T, I, gated, act, (const bf16*)pre,
+                       (const bf16*)dhid, (bf16*)dpre);
+  else if (dtype == LT_F32)
     hipLaunchKernelGGL((act_bwd_kernel<float>), grid, block, 0, stream, T, I, gated, act, (const float*)pre,
                        (const float*)dhid, (float*)dpre);
   else
