@@ -253,7 +253,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       else b[j] = frag_mn(lds_b[s], std::integral_constant<int, BN>{}, wn * WTN + j * 32, kk);
     }
   };
-  constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);  // LDS read instructions per k-substep
+  constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);
+  // LDS reads of a half-step spread over this many of its 16 matrix instructions: evenly over all of them, except for the
+  // mixed layout, which measured 2 % faster with the reads done by the twelfth
+  constexpr int READ_SPAN = (A_KM && !B_KM) ? 12 : 16;  // LDS read instructions per k-substep
 
   // split-k: this workgroup's slice of the k-steps
   int kt_begin = 0, kt_end = kt_total;
@@ -465,14 +468,17 @@ constexpr int DK = 32;  // k per step of the copy-based kernel
 
 // scheduling hint for one half k-step: READS LDS reads and COPIES global->LDS copies spread evenly over MFMAS matrix
 // instructions (packing the reads into the first half of the matrix instructions measured slower)
-template <int READS, int COPIES, int MFMAS, int G = 0> struct SchedInterleave3 {
+template <int READS, int COPIES, int MFMAS, int READ_SPAN, int G = 0> struct SchedInterleave3 {
   static __device__ __forceinline__ void run() {
-    constexpr int nr = READS * (G + 1) / MFMAS - READS * G / MFMAS;
+    // the LDS reads go out over the first SPAN matrix instructions, the copies over all of them
+    constexpr int SPAN = READ_SPAN < MFMAS ? READ_SPAN : MFMAS;
+    constexpr int g0 = G < SPAN ? G : SPAN, g1 = G + 1 < SPAN ? G + 1 : SPAN;
+    constexpr int nr = READS * g1 / SPAN - READS * g0 / SPAN;
     constexpr int nc = COPIES * (G + 1) / MFMAS - COPIES * G / MFMAS;
     if constexpr (nr > 0) __builtin_amdgcn_sched_group_barrier(0x100, nr, 0);
     if constexpr (nc > 0) __builtin_amdgcn_sched_group_barrier(0x020, nc, 0);
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    if constexpr (G + 1 < MFMAS) SchedInterleave3<READS, COPIES, MFMAS, G + 1>::run();
+    if constexpr (G + 1 < MFMAS) SchedInterleave3<READS, COPIES, MFMAS, READ_SPAN, G + 1>::run();
   }
 };
 
@@ -481,15 +487,9 @@ template <int READS, int COPIES, int MFMAS, int G = 0> struct SchedInterleave3 {
 // that older copies have landed; the empty asm statements only keep it from moving LDS accesses across the barrier.
 template <int N> __device__ __forceinline__ void wait_copies_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-#ifdef LT_DBG_NO_WAIT
-  __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));
-#else
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));  // vmcnt(N) expcnt(7: none) lgkmcnt(0)
-#endif
   asm volatile("" ::: "memory");
-#ifndef LT_DBG_NO_BARRIER
   __builtin_amdgcn_s_barrier();
-#endif
   asm volatile("" ::: "memory");
 }
 
@@ -588,18 +588,10 @@ static_assert(copies_in_flight(false, false, {}, {}, false, 0) == 16 && copies_i
               copies_in_flight(true, true, {{0, 0}}, {{1, 1}}, false, 1) == 0 && copies_in_flight(false, false, {}, {}, true, 0) == 12,
               "issue-order model");
 
-#ifndef LT_NT_A
-#define LT_NT_A {0, 0}
-#endif
-#ifndef LT_NT_B
-#define LT_NT_B {2, 2}
-#endif
-#ifndef LT_NN_A
-#define LT_NN_A {0, 2}
-#endif
-#ifndef LT_B_SPLIT
-#define LT_B_SPLIT 1
-#endif
+// Measured choices (config-3 GEMM shapes): two k-major operands -- A block right after the odd barrier, B block after the
+// even one; k-major A next to mn-major B -- A split over both barriers; two mn-major operands -- B in the second half-step.
+constexpr BlockSlots SLOTS_NT_A = {{0, 0}}, SLOTS_NT_B = {{2, 2}}, SLOTS_NN_A = {{0, 2}};
+constexpr bool SPLIT_MN_B = true;
 
 template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
@@ -755,6 +747,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     }
   };
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);
+  // LDS reads of a half-step spread over this many of its 16 matrix instructions: evenly over all of them, except for the
+  // mixed layout, which measured 2 % faster with the reads done by the twelfth
+  constexpr int READ_SPAN = (A_KM && !B_KM) ? 12 : 16;
   constexpr int N_MN = (A_KM ? 0 : 4) + (B_KM ? 0 : 4);  // copy instructions per k-step for the mn-major operands
   constexpr int N_KM = (A_KM ? 8 : 0) + (B_KM ? 8 : 0);  // copy instructions per block for the k-major operands
 
@@ -769,8 +764,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   // Copies are spread over the half-steps so that the address unit, which the four wavefronts share, is not handed whole
   // blocks at once: the halves of a k-major block go out in the slots of SA / SB, mn-major B (next to mn-major A) in the
   // second half of every k-step (B_SPLIT); the rest in the first half.
-  constexpr BlockSlots SA = B_KM ? BlockSlots{LT_NT_A} : BlockSlots{LT_NN_A}, SB = BlockSlots{LT_NT_B};
-  constexpr bool B_SPLIT = !B_KM && !A_KM && LT_B_SPLIT;
+  constexpr BlockSlots SA = B_KM ? SLOTS_NT_A : SLOTS_NN_A, SB = SLOTS_NT_B;
+  constexpr bool B_SPLIT = !B_KM && !A_KM && SPLIT_MN_B;
   using J0 = std::integral_constant<int, 0>;
   using J4 = std::integral_constant<int, 4>;
   using J8 = std::integral_constant<int, 8>;
@@ -803,7 +798,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 #pragma unroll
       for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][x], bfr[0][y], acc[x][y], 0, 0, 0);
     constexpr int COPIES = (A_KM ? 0 : 4) + ((B_KM || B_SPLIT) ? 0 : 4) + ((i & 1) == 0 ? slot_copies(1) : 0);
-    SchedInterleave3<FRAG_READS, COPIES, FM * FN>::run();
+    SchedInterleave3<FRAG_READS, COPIES, FM * FN, READ_SPAN>::run();
   };
   auto second_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
@@ -829,7 +824,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 #pragma unroll
       for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][x], bfr[1][y], acc[x][y], 0, 0, 0);
     constexpr int COPIES = (B_SPLIT ? 4 : 0) + (N_KM > 0 ? slot_copies((i & 1) ? 0 : 2) : 0);
-    SchedInterleave3<FRAG_READS, COPIES, FM * FN>::run();
+    SchedInterleave3<FRAG_READS, COPIES, FM * FN, READ_SPAN>::run();
   };
   using Steady = std::integral_constant<bool, true>;
   using Ragged = std::integral_constant<bool, false>;
