@@ -5,13 +5,16 @@
 namespace {
 
 constexpr int LN_MAXV = 32;  // float4 per lane held in registers: rows up to 64 * 4 * 32 = 8192 elements stay on chip
+// The row kernels are instantiated for 8, 16 and 32 vectors per lane (hidden <= 2048, 4096, 8192): the register arrays are
+// sized by the template argument, so a narrower row leaves room for more wavefronts per SIMD.
+static int ln_vectors_per_lane(int H) { return H <= 2048 ? 8 : H <= 4096 ? 16 : 32; }
 
 // ---------------------------------------------------------------------------------------------------------------------
 // LayerNorm forward: one wavefront per row.  The row is read once into registers (when hidden % 4 == 0 and it fits), the
 // mean and the centred second moment are reduced across the 64 lanes with shuffles, and the normalised row is written in
 // the GEMM operand dtype.  TAIL fuses what follows a post-LayerNorm: dropout, then the residual add.
 // ---------------------------------------------------------------------------------------------------------------------
-template <typename TX, typename TY, typename TR, bool TAIL>
+template <typename TX, typename TY, typename TR, bool TAIL, int MAXV>
 __global__ __launch_bounds__(256) void ln_fwd_kernel(int64_t T, int H, float eps, const TX* __restrict__ x,
                                                       const float* __restrict__ w, const float* __restrict__ b,
                                                       TY* __restrict__ y, float* __restrict__ stats,
@@ -23,10 +26,10 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(int64_t T, int H, float eps
   const float inv_h = 1.0f / (float)H;
   float mean, rstd;
   if (vec) {
-    float v[LN_MAXV][4];
+    float v[MAXV][4];
     float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < LN_MAXV; i++) {
+    for (int i = 0; i < MAXV; i++) {
       const int c = (i * 64 + lane) * 4;
       if (c < H) {
         load4(xr + c, v[i]);
@@ -36,7 +39,7 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(int64_t T, int H, float eps
     mean = wave_sum(s) * inv_h;
     float q = 0.f;
 #pragma unroll
-    for (int i = 0; i < LN_MAXV; i++) {
+    for (int i = 0; i < MAXV; i++) {
       const int c = (i * 64 + lane) * 4;
       if (c < H) {
 #pragma unroll
@@ -49,7 +52,7 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(int64_t T, int H, float eps
     rstd = 1.0f / sqrtf(wave_sum(q) * inv_h + eps);
     if (y) {
 #pragma unroll
-      for (int i = 0; i < LN_MAXV; i++) {
+      for (int i = 0; i < MAXV; i++) {
         const int c = (i * 64 + lane) * 4;
         if (c < H) {
           float wv[4], bv[4], o[4];
@@ -185,7 +188,7 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(int64_t T, int H, const TX*
 //                         shuffles, dx (+ residual gradient) is written with 16-byte stores
 //   ln_bwd_param_kernel   column-parallel: 64 lanes x 4 columns per workgroup and 4 row lanes walking a slice of rows;
 //                         writes one partial (dweight, dbias) row per slice, summed by colreduce_kernel
-template <typename TX, typename TDY, typename TDX>
+template <typename TX, typename TDY, typename TDX, int MAXV>
 __global__ __launch_bounds__(256) void ln_bwd_dx_kernel(int64_t T, int H, const TX* __restrict__ x,
                                                          const float* __restrict__ stats, const float* __restrict__ w,
                                                          const TDY* __restrict__ dy, const TDX* __restrict__ residual_grad,
@@ -196,10 +199,10 @@ __global__ __launch_bounds__(256) void ln_bwd_dx_kernel(int64_t T, int H, const 
   const float mean = stats[row * 2], rstd = stats[row * 2 + 1];
   const TX* xr = x + row * H;
   const TDY* dyr = dy + row * H;
-  float xh[LN_MAXV][4], dxh[LN_MAXV][4];
+  float xh[MAXV][4], dxh[MAXV][4];
   float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-  for (int i = 0; i < LN_MAXV; i++) {
+  for (int i = 0; i < MAXV; i++) {
     const int c = (i * 64 + lane) * 4;
     if (c < H) {
       float wv[4];
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(256) void ln_bwd_dx_kernel(int64_t T, int H, const 
   const float inv_h = 1.0f / (float)H;
   const float c1 = wave_sum(s1) * inv_h, c2 = wave_sum(s2) * inv_h;
 #pragma unroll
-  for (int i = 0; i < LN_MAXV; i++) {
+  for (int i = 0; i < MAXV; i++) {
     const int c = (i * 64 + lane) * 4;
     if (c < H) {
       float o[4];
@@ -565,9 +568,16 @@ int lt_ln_forward(int64_t T, int H, float eps, int x_dtype, const void* x, const
                        (double)T * H * (lt_dtype_size(x_dtype) + (y ? lt_dtype_size(y_dtype) : 0) +
                                         (residual ? lt_dtype_size(res_dtype) : 0)) + (stats ? 8.0 * T : 0.0),
                        stream);
-#define LT_LN_LAUNCH(TX, TY, TR, TAILV)                                                                              \
-  hipLaunchKernelGGL((ln_fwd_kernel<TX, TY, TR, TAILV>), grid, block, 0, stream, T, H, eps, (const TX*)x, w, b, (TY*)y, \
+  const int maxv = ln_vectors_per_lane(H);
+#define LT_LN_LAUNCH_V(TX, TY, TR, TAILV, MAXV)                                                                             \
+  hipLaunchKernelGGL((ln_fwd_kernel<TX, TY, TR, TAILV, MAXV>), grid, block, 0, stream, T, H, eps, (const TX*)x, w, b, (TY*)y, \
                      stats, (const TR*)residual, d, vec)
+#define LT_LN_LAUNCH(TX, TY, TR, TAILV)                     \
+  do {                                                      \
+    if (maxv == 8) LT_LN_LAUNCH_V(TX, TY, TR, TAILV, 8);    \
+    else if (maxv == 16) LT_LN_LAUNCH_V(TX, TY, TR, TAILV, 16); \
+    else LT_LN_LAUNCH_V(TX, TY, TR, TAILV, 32);             \
+  } while (0)
   if (!tail) {
     if (x_dtype == LT_F32 && y_dtype == LT_F32) LT_LN_LAUNCH(float, float, float, false);
     else if (x_dtype == LT_F32) LT_LN_LAUNCH(float, bf16, float, false);
@@ -582,6 +592,7 @@ int lt_ln_forward(int64_t T, int H, float eps, int x_dtype, const void* x, const
     else LT_LN_LAUNCH(bf16, bf16, bf16, true);
   }
 #undef LT_LN_LAUNCH
+#undef LT_LN_LAUNCH_V
   LT_LAUNCH_CHECK();
   return LT_OK;
 }
@@ -622,9 +633,16 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   if (vec) {
     if (dx) {
       dim3 grid(blocks_for(T, 4)), block(256);
-#define LT_LNB_DX(TX, TDY, TDX)                                                                                         \
-  hipLaunchKernelGGL((ln_bwd_dx_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
+      const int maxv = ln_vectors_per_lane(H);
+#define LT_LNB_DX_V(TX, TDY, TDX, MAXV)                                                                                       \
+  hipLaunchKernelGGL((ln_bwd_dx_kernel<TX, TDY, TDX, MAXV>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
                      (const TDX*)residual_grad, (TDX*)dx)
+#define LT_LNB_DX(TX, TDY, TDX)                        \
+  do {                                                 \
+    if (maxv == 8) LT_LNB_DX_V(TX, TDY, TDX, 8);       \
+    else if (maxv == 16) LT_LNB_DX_V(TX, TDY, TDX, 16); \
+    else LT_LNB_DX_V(TX, TDY, TDX, 32);                \
+  } while (0)
       switch (key) {
         case 0: LT_LNB_DX(float, float, float); break;
         case 1: LT_LNB_DX(float, float, bf16); break;
@@ -636,6 +654,7 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
         default: LT_LNB_DX(bf16, bf16, bf16); break;
       }
 #undef LT_LNB_DX
+#undef LT_LNB_DX_V
       LT_LAUNCH_CHECK();
     }
     partial_rows = ln_bwd_slices(T);
