@@ -135,8 +135,12 @@ void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, 
   s.colsum_bytes = lt_colsum_workspace(T, lin.out_features);
   s.colsum = ws.take(s.colsum_bytes);
   s.skinny_bytes = lin.lowrank > 0 ? lt_gemm_skinny_workspace(T, lin.lowrank) : 0;
-  if (lin.block == 0 && dtype == LT_BF16)  // dW of a small dense layer: reduction over the tokens split across workgroups
+  if (lin.block == 0) {  // dW (and dx) of a small dense layer: the reduction is split across workgroups
     s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_splitk_workspace(lin.out_features, lin.in_features, T));
+    s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_generic_splitk_workspace(lin.out_features, lin.in_features, T));
+    if (lin.lowrank == 0)
+      s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_generic_splitk_workspace(T, lin.in_features, lin.out_features));
+  }
   s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 
@@ -176,7 +180,8 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
         p.epi.colsum = act_colsum;
         *act_colsum_done = true;
       }
-      LT_TRY(lt_launch_gemm(p, kind_dx, dtype, io_dtype, stream));
+      if (kind_dx == EPI_STORE && r == 0) LT_TRY(lt_launch_gemm_skinny(p, dtype, io_dtype, s.skinny, s.skinny_bytes, stream));
+      else LT_TRY(lt_launch_gemm(p, kind_dx, dtype, io_dtype, stream));
     } else {
       p.K[0] = lin.block;
       p.sp.mode = SPARSE_DX; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;

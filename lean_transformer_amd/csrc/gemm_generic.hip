@@ -111,6 +111,14 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmProblem p) {
   int seg = 0;
   Segment<TI> g = segment(0);
   int64_t k0 = 0;
+  if (sp.mode == SPARSE_NONE && p.ksplit > 1) {
+    // split reduction (one k-segment, EPI_STORE): slice blockIdx.z walks a whole number of k-steps and stores fp32 partial
+    // sums at epi.out + slice * split_stride
+    const int64_t steps = (g.K + GBK - 1) / GBK, per = (steps + p.ksplit - 1) / p.ksplit * GBK;
+    k0 = min(g.K, (int64_t)blockIdx.z * per);
+    g.K = min(g.K, k0 + per);
+    epi.out = reinterpret_cast<float*>(epi.out) + (int64_t)blockIdx.z * p.split_stride;
+  }
   auto fetch = [&](Fetch& f) {
     // A: k-major -> 4 consecutive k of one row; mn-major -> 4 consecutive rows of one k
     const bool va = (reinterpret_cast<uintptr_t>(g.A) % (4 * sizeof(TI)) == 0) && (g.lda & 3) == 0 &&
@@ -198,7 +206,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmProblem p) {
   };
 
   Fetch f;
-  fetch(f);
+  fetch(f);  // an empty slice (k0 == K) fetches zeros
   stash(f, 0);
   __syncthreads();
   int buf = 0;
@@ -310,6 +318,11 @@ int lt_launch_gemm_generic(const GemmProblem& p, int kind, int dtype, int io_dty
   }
   static const char* tags[4] = {"gemm_generic", "blocksparse_fwd_generic", "blocksparse_dx_generic", "blocksparse_dw_generic"};
   LtProfileScope scope(tags[sp.mode], flops, 0.0, stream);
+  if (sp.mode == SPARSE_NONE && p.ksplit > 1) {
+    LT_REQUIRE(kind == EPI_STORE && p.nseg == 1 && p.epi.out_dtype == LT_F32 && !p.epi.bias, LT_ERR_BAD_ARG,
+               "gemm: a split reduction stores fp32 partial sums of one k-segment");
+    groups = p.ksplit;
+  }
   dim3 grid((unsigned)tiles_n, (unsigned)tiles_m, (unsigned)groups);
   return dtype == LT_F32 ? launch_kind<float>(p, kind, io_dtype, grid, stream)
                          : launch_kind<bf16>(p, kind, io_dtype, grid, stream);

@@ -1308,6 +1308,20 @@ size_t lt_gemm_splitk_workspace(int64_t M, int64_t N, int64_t K) {
   return slices > 1 ? lt_align_up((size_t)slices * (size_t)M * (size_t)N * sizeof(float), 256) : 0;
 }
 
+namespace {
+// the any-shape kernel runs four 128 x 128 workgroups per CU: slices of at least eight k-steps until about 1024 workgroups
+int generic_splitk_slices(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles >= 768) return 1;
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(1024 / tiles, K / 128), 16));
+}
+}  // namespace
+
+size_t lt_gemm_generic_splitk_workspace(int64_t M, int64_t N, int64_t K) {
+  const int slices = generic_splitk_slices(M, N, K);
+  return slices > 1 ? lt_align_up((size_t)slices * (size_t)M * (size_t)N * sizeof(float), 256) : 0;
+}
+
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                           hipStream_t stream) {
   const bool a_km = p.A[0].kmajor, b_km = p.B[0].kmajor;
@@ -1335,7 +1349,24 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
     }
     if (((p.M + 255) / 256) * (p.N / 256) >= 64 || slices == 1) ok = false;
   }
-  if (!ok) return lt_launch_gemm(p, EPI_STORE, dtype, io_dtype, stream);
+  if (!ok) {
+    // any-shape kernel: split the reduction when the tiles alone leave most workgroup slots empty
+    const bool tiled = dtype == LT_BF16 && lt_gemm_mfma_supported(p, EPI_STORE);
+    const int slices = (!tiled && p.nseg == 1 && p.sp.mode == SPARSE_NONE && e.ldo == p.N && (p.N & 3) == 0 &&
+                        lt_aligned(e.out, 16) && (!e.bias || lt_aligned(e.bias, 16)))
+                           ? generic_splitk_slices(p.M, p.N, p.K[0]) : 1;
+    if (slices > 1 && workspace && workspace_bytes >= (size_t)slices * (size_t)p.M * (size_t)p.N * sizeof(float)) {
+      GemmProblem q = p;
+      q.ksplit = slices;
+      q.split_stride = p.M * p.N;
+      q.epi.out = workspace;
+      q.epi.out_dtype = LT_F32;
+      q.epi.bias = nullptr;
+      LT_TRY(lt_launch_gemm_generic(q, EPI_STORE, dtype, io_dtype, stream));
+      return lt_splitk_reduce((const float*)workspace, slices, p.M * p.N, p.M * p.N, (int)p.N, e.bias, e.out_dtype, e.out, stream);
+    }
+    return lt_launch_gemm(p, EPI_STORE, dtype, io_dtype, stream);
+  }
   const int kt_total = (int)((p.K[0] + BK - 1) / BK);
   int slices = 1;
   if (workspace && tiles < 192) {

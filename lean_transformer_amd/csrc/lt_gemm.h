@@ -450,6 +450,8 @@ int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtyp
 size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank);
 // partial sums of a split [M, N] result on 256 x 256 tiles (0 when the tiles alone fill the chip)
 size_t lt_gemm_splitk_workspace(int64_t M, int64_t N, int64_t K);
+// same for the any-shape kernel (fp32 path, shapes the tiled kernels do not take)
+size_t lt_gemm_generic_splitk_workspace(int64_t M, int64_t N, int64_t K);
 // true when lt_launch_gemm sends this EPI_ACT_BWD problem to the kernel that fills EpiParams::colsum
 bool lt_gemm_fuses_colsum(const GemmProblem& p, int dtype, int io_dtype);
 // out[c] = sum over `rows` partial rows of partial[r * stride + c]
