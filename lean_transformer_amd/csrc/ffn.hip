@@ -147,12 +147,13 @@ void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, 
 // gradient side of one generalized linear layer.  The input-gradient GEMM runs FIRST, through epilogue `kind_dx`
 // (EPI_ACT_BWD for the down-projection, whose epilogue also re-materialises this layer's own input `x_act`), then the
 // parameter gradients, which may therefore read x_act.  Pass kind_dx < 0 to skip the input gradient.
-// act_colsum / act_colsum_done: with an EPI_ACT_BWD input-gradient epilogue, room for the partial column sums of the dpre it
-// writes (one row of epi_dx.ld_pre floats per 128 tokens); *act_colsum_done says whether the kernel that ran filled it
+// act_colsum / act_colsum_rows: with an EPI_ACT_BWD input-gradient epilogue, room for the partial column sums of the dpre it
+// writes (one row of epi_dx.ld_pre floats per 64 tokens); *act_colsum_rows = tokens per partial row the kernel that ran
+// filled (0: it did not)
 int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void* x_act, const void* dy,
                          const void* lowrank_hid, int kind_dx, const EpiParams& epi_dx, const lt_linear_grads& grads,
                          const LinearBwdScratch& s, int io_dtype, hipStream_t stream, float* act_colsum = nullptr,
-                         bool* act_colsum_done = nullptr) {
+                         int* act_colsum_rows = nullptr) {
   const int64_t in = lin.in_features, out = lin.out_features, r = lin.lowrank;
   const bool need_dx = kind_dx >= 0;
   if (r > 0 && (need_dx || grads.lowrank_first)) {  // g_hid = dy L2  [T, r]
@@ -176,10 +177,8 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.K[0] = out;
       p.A[0] = operand(dy, out, true);
       p.B[0] = operand(lin.weight, in, false);
-      if (kind_dx == EPI_ACT_BWD && act_colsum && lt_gemm_fuses_colsum(p, dtype, io_dtype)) {
+      if (kind_dx == EPI_ACT_BWD && act_colsum && (*act_colsum_rows = lt_gemm_colsum_rows(p, dtype, io_dtype)) > 0)
         p.epi.colsum = act_colsum;
-        *act_colsum_done = true;
-      }
       if (kind_dx == EPI_STORE && r == 0) LT_TRY(lt_launch_gemm_skinny(p, dtype, io_dtype, s.skinny, s.skinny_bytes, stream));
       else LT_TRY(lt_launch_gemm(p, kind_dx, dtype, io_dtype, stream));
     } else {
@@ -187,6 +186,8 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.mode = SPARSE_DX; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
       p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.weight = lin.weight;
+      if (kind_dx == EPI_ACT_BWD && act_colsum && (*act_colsum_rows = lt_gemm_colsum_rows(p, dtype, io_dtype)) > 0)
+        p.epi.colsum = act_colsum;
       LT_TRY(lt_launch_gemm_sparse(p, kind_dx, dtype, io_dtype, stream));
     }
   }
@@ -275,7 +276,7 @@ struct BwdScratch {
   float* du;         // [T, H] fp32
   void* ln_ws;
   size_t ln_ws_bytes;
-  float* act_colsum;  // [ceil(T / 128), N1]: partial column sums of dpre from the epilogue that writes it
+  float* act_colsum;  // [ceil(T / 64), N1]: partial column sums of dpre from the epilogue that writes it
   LinearBwdScratch h2o, i2h;
 };
 
@@ -292,7 +293,7 @@ void plan_backward(const lt_ffn_desc& d, Bump& ws, BwdScratch& s) {
   s.du = (float*)ws.take((size_t)T * d.hidden * sizeof(float));
   s.ln_ws_bytes = lt_ln_backward_workspace(T, d.hidden);
   s.ln_ws = ws.take(s.ln_ws_bytes);
-  s.act_colsum = (float*)ws.take((size_t)((T + 127) / 128) * n1 * sizeof(float));
+  s.act_colsum = (float*)ws.take((size_t)((T + 63) / 64) * n1 * sizeof(float));
   plan_linear_backward(d.h2o, T, d.compute_dtype, ws, s.h2o);
   plan_linear_backward(d.i2h, T, d.compute_dtype, ws, s.i2h);
 }
@@ -408,18 +409,18 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   }
 
   // down-projection backward; its input-gradient epilogue turns dh into dP and re-materialises h from P
-  bool bias_from_epilogue = false;
+  int bias_rows = 0;  // tokens per partial row of s.act_colsum when the dGeGLU epilogue summed the columns of dP
   {
     EpiParams e;
     memset(&e, 0, sizeof(e));
     e.pre = saved->pre_activation; e.ld_pre = N1; e.dpre = s.dpre; e.hid = s.hid; e.ld_hid = I;
     e.gated = d.gated; e.act = d.act; e.inter = I;
     LT_TRY(linear_backward_impl(d.h2o, T, cdt, s.hid, g, saved->h2o_lowrank_hid, EPI_ACT_BWD, e, h2o_grads, s.h2o, io,
-                                stream, grads->i2h.bias ? s.act_colsum : nullptr, &bias_from_epilogue));
+                                stream, grads->i2h.bias ? s.act_colsum : nullptr, &bias_rows));
   }
   lt_linear_grads i2h_grads = grads->i2h;
-  if (bias_from_epilogue) {  // db1 = column sums of dP, already reduced to one row per 128 tokens
-    LT_TRY(lt_colreduce((int)((T + 127) / 128), N1, (int)N1, s.act_colsum, (float*)grads->i2h.bias, stream));
+  if (bias_rows > 0) {  // db1 = column sums of dP, already reduced to one row per bias_rows tokens
+    LT_TRY(lt_colreduce((int)((T + bias_rows - 1) / bias_rows), N1, (int)N1, s.act_colsum, (float*)grads->i2h.bias, stream));
     i2h_grads.bias = nullptr;
   }
 

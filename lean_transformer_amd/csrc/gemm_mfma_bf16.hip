@@ -394,10 +394,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     }
     __builtin_amdgcn_wave_barrier();
   };
+  float colsum[16];  // EPI_ACT_BWD: column sums of this lane's 8 (+ 8) dpre columns over the rows it writes
+#pragma unroll
+  for (int e = 0; e < 16; e++) colsum[e] = 0.f;
   auto act_bwd_strip = [&](auto I, auto G) __attribute__((always_inline)) {
     constexpr int i = decltype(I)::value;
     constexpr bool GATED = decltype(G)::value;
-    float unused[16];
     EpiLoad rows[NIT];
 #pragma unroll
     for (int it = 0; it < NIT; it++) rows[it] = epi_load_pre8<GATED>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n);
@@ -406,7 +408,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     for (int it = 0; it < NIT; it++) {
       float v[8];
       read_staged(it, v);
-      epi_act_bwd8_gelu<GATED>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n, v, rows[it], unused);
+      epi_act_bwd8_gelu<GATED>(epi, lane_row(i) + it * ROWS_PER_IT, lane_n, v, rows[it], colsum);
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -434,6 +436,27 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     if (straight && epi.gated) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { act_bwd_strip(I, std::true_type{}); });
     else if (straight) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { act_bwd_strip(I, std::false_type{}); });
     else lt_static_for<FM>(generic_strip);
+    if (straight && epi.colsum) {
+      // lanes with equal lane % LANES_PER_ROW hold the same columns for different rows of the wavefront's WTM-row sub-tile:
+      // one partial row per wavefront sub-tile
+      static_assert(WTM == 64 || KIND != EPI_ACT_BWD || NIT > 4, "the caller reduces one partial row per 64 output rows");
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+#pragma unroll
+        for (int d = LANES_PER_ROW; d < 64; d <<= 1) colsum[e] += __shfl_xor(colsum[e], d);
+      }
+      if (lane < LANES_PER_ROW) {
+        float* dst = epi.colsum + ((m_base + wm * WTM) / 64) * epi.ld_pre + lane_n;
+        float lo[8], hi[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          lo[e] = colsum[e];
+          hi[e] = colsum[8 + e];
+        }
+        store8(dst, lo);
+        if (epi.gated) store8(dst + epi.inter, hi);
+      }
+    }
   } else if constexpr (NIT <= 4 && KIND == EPI_OUT) {
     if (whole_tile && epi.x && epi.drop.p == 0.f) lt_static_for<FM>(out_strip);
     else lt_static_for<FM>(generic_strip);
@@ -1242,9 +1265,16 @@ bool lt_gemm_mfma_supported(const GemmProblem& p, int kind) {
   return true;
 }
 
-bool lt_gemm_fuses_colsum(const GemmProblem& p, int dtype, int io_dtype) {
-  return dtype == LT_BF16 && p.sp.mode == SPARSE_NONE && lt_gemm_mfma_supported(p, EPI_ACT_BWD) &&
-         dma_selected(p, EPI_ACT_BWD, io_dtype) && p.epi.ld_pre % 8 == 0;
+bool lt_sparse_mfma_supported(const GemmProblem& p, int kind);
+
+int lt_gemm_colsum_rows(const GemmProblem& p, int dtype, int io_dtype) {
+  if (dtype != LT_BF16 || p.epi.ld_pre % 8 != 0) return 0;
+  if (p.sp.mode == SPARSE_NONE)
+    return lt_gemm_mfma_supported(p, EPI_ACT_BWD) && dma_selected(p, EPI_ACT_BWD, io_dtype) ? 128 : 0;
+  // the walk's straight-line strips keep the sums: every tile must take them
+  return p.sp.mode == SPARSE_DX && lt_sparse_mfma_supported(p, EPI_ACT_BWD) && p.M % 256 == 0 &&
+                 p.epi.act == LT_ACT_GELU_FUSED && p.epi.hid
+             ? 64 : 0;
 }
 
 static const char* mfma_tag(const GemmProblem& p, int kind) {

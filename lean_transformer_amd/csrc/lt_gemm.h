@@ -32,8 +32,8 @@ struct EpiParams {
   int gated;
   int act;
   int64_t inter;      // I
-  // ACT_BWD on the copy-based kernel only (see lt_gemm_fuses_colsum): column sums of the dpre values as stored, one partial
-  // row per 128 rows of the output: colsum[(m / 128) * ld_pre + column].  Null = off.
+  // ACT_BWD where lt_gemm_colsum_rows says so: column sums of the dpre values as stored, one partial row per R rows of the
+  // output (R = that function's result): colsum[(m / R) * ld_pre + column].  Null = off.
   float* colsum;
   // EPI_OUT
   const void* x;      // residual input [M, ldy] (null = no residual)
@@ -452,8 +452,9 @@ size_t lt_gemm_skinny_workspace(int64_t tokens, int64_t lowrank);
 size_t lt_gemm_splitk_workspace(int64_t M, int64_t N, int64_t K);
 // same for the any-shape kernel (fp32 path, shapes the tiled kernels do not take)
 size_t lt_gemm_generic_splitk_workspace(int64_t M, int64_t N, int64_t K);
-// true when lt_launch_gemm sends this EPI_ACT_BWD problem to the kernel that fills EpiParams::colsum
-bool lt_gemm_fuses_colsum(const GemmProblem& p, int dtype, int io_dtype);
+// rows per partial row of EpiParams::colsum when lt_launch_gemm / lt_launch_gemm_sparse sends this EPI_ACT_BWD problem to a
+// kernel that fills it (128: copy-based dense kernel; 64: block-sparse walk on whole tiles with the tanh GELU); 0: it will not
+int lt_gemm_colsum_rows(const GemmProblem& p, int dtype, int io_dtype);
 // out[c] = sum over `rows` partial rows of partial[r * stride + c]
 int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream);
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
