@@ -253,10 +253,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       else b[j] = frag_mn(lds_b[s], std::integral_constant<int, BN>{}, wn * WTN + j * 32, kk);
     }
   };
-  constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);
-  // LDS reads of a half-step spread over this many of its 16 matrix instructions: evenly over all of them, except for the
-  // mixed layout, which measured 2 % faster with the reads done by the twelfth
-  constexpr int READ_SPAN = (A_KM && !B_KM) ? 12 : 16;  // LDS read instructions per k-substep
+  constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);  // LDS read instructions per k-substep
 
   // split-k: this workgroup's slice of the k-steps
   int kt_begin = 0, kt_end = kt_total;
