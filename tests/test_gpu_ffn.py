@@ -222,6 +222,53 @@ def test_ffn_bf16_tiled_kernels_against_cpu_oracle(gated, tokens, io_dtype):
     _compare(ffn, x, dy, torch.bfloat16)
 
 
+@pytest.mark.parametrize("tokens", [257, 513])
+def test_ffn_bf16_one_row_past_a_tile(tokens):
+    """a launch whose last 256-row tile holds a single row: whole tiles take the straight-line epilogue strips, the last one
+    the general strips, and the fused column sums (bias gradients) must cover exactly the rows that exist"""
+    torch.manual_seed(tokens)
+    ffn = lt.LeanFFN(512, 1024, gated=True, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.i2h_proj.bias.normal_(std=0.1)
+        ffn.h2o_proj.bias.normal_(std=0.1)
+    ffn = ffn.to(DEV).to(torch.bfloat16)
+    x, dy = torch.randn(tokens, 512), torch.randn(tokens, 512)
+    _compare(ffn, x, dy, torch.bfloat16)
+
+
+@pytest.mark.parametrize("hidden,inter", [(192, 320), (264, 520)])
+def test_ffn_bf16_sizes_off_the_tile_grid(hidden, inter):
+    """bf16 weights with hidden / intermediate sizes the 256-wide tiles do not divide: the any-shape kernel on bf16 operands"""
+    torch.manual_seed(hidden)
+    ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5).to(DEV).to(torch.bfloat16)
+    x, dy = torch.randn(300, hidden), torch.randn(300, hidden)
+    _compare(ffn, x, dy, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ffn_empty_batch(dtype):
+    """zero tokens: output and input gradient are empty, parameter gradients are zeros (the reference's stock ops agree)"""
+    ffn = lt.LeanFFN(256, 512, gated=True).to(DEV).to(dtype)
+    x = torch.zeros(0, 256, device=DEV, dtype=dtype, requires_grad=True)
+    y = ffn(x)
+    assert y.shape == (0, 256)
+    grads = torch.autograd.grad(y, [x, *ffn.parameters()], torch.zeros_like(y))
+    assert grads[0].shape == (0, 256)
+    for g, prm in zip(grads[1:], ffn.parameters()):
+        assert g.shape == prm.shape and g.dtype == prm.dtype and not g.any()
+
+
+def test_ffn_refuses_what_it_cannot_run():
+    """loud failures, no fallback: half precision, an activation the kernels do not have, a plug-in matmul op"""
+    ffn = lt.LeanFFN(256, 512).to(DEV)
+    with pytest.raises(TypeError):
+        ffn.half()(torch.zeros(4, 256, device=DEV, dtype=torch.float16))
+    with pytest.raises((NotImplementedError, ValueError, KeyError, RuntimeError)):
+        lt.LeanFFN(256, 512, activation=lambda t: t * 2).to(DEV)(torch.zeros(4, 256, device=DEV))
+    with pytest.raises(RuntimeError):
+        lt.LeanFFN(256, 512).to(DEV)(torch.zeros(4, 128, device=DEV))
+
+
 def test_ffn_autocast_fp32_master_weights():
     """fp32 parameters under torch.autocast(bfloat16): GEMM operands are cast per call, gradients come back in fp32"""
     torch.manual_seed(5)
