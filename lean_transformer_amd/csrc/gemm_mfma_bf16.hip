@@ -1055,7 +1055,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     }
     __builtin_amdgcn_wave_barrier();
   };
-  auto out_strip = [&](auto I) {
+  auto out_strip = [&](auto I, auto D) {
+    constexpr bool DROPOUT = decltype(D)::value;
     constexpr int i = decltype(I)::value;
     constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
     const int c = (lane % LANES_PER_ROW) * 8;
@@ -1071,7 +1072,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       const float* sv = staged(it * ROWS_PER_IT + lane / LANES_PER_ROW, c);
 #pragma unroll
       for (int e = 0; e < 8; e++) v[e] = sv[e];
-      epi_out8_residual<TX>(epi, mlane + it * ROWS_PER_IT, n, v, win[it % ACT_WINDOW]);
+      epi_out8_residual<TX, DROPOUT>(epi, mlane + it * ROWS_PER_IT, n, v, win[it % ACT_WINDOW]);
       if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_x8<TX>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
     }
     __builtin_amdgcn_wave_barrier();
@@ -1092,7 +1093,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     else for_each_strip(generic_strip);
   } else {
     if (whole_tile && epi.x && epi.drop.p == 0.f) {
-      for_each_strip(out_strip);
+      for_each_strip([&](auto I) { out_strip(I, std::false_type{}); });
+    } else if (whole_tile && epi.x) {
+      for_each_strip([&](auto I) { out_strip(I, std::true_type{}); });
     } else {
       for_each_strip(generic_strip);
     }

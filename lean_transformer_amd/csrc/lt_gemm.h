@@ -340,8 +340,20 @@ template <typename TX> __device__ __forceinline__ EpiLoad epi_load_x8(const EpiP
   return l;
 }
 
-template <typename TX>
+// DROPOUT: Philox keep-mask of the 8 elements applied before the residual is added
+template <typename TX, bool DROPOUT = false>
 __device__ __forceinline__ void epi_out8_residual(const EpiParams& e, int64_t m, int64_t n, float (&v)[8], const EpiLoad& l) {
+  if constexpr (DROPOUT) {
+    const int64_t idx = m * e.ldy + n;
+    bool k0[4], k1[4];
+    dropout_keep4(e.drop, idx, k0);
+    dropout_keep4(e.drop, idx + 4, k1);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[i] = k0[i] ? v[i] * e.drop.scale : 0.f;
+      v[i + 4] = k1[i] ? v[i + 4] * e.drop.scale : 0.f;
+    }
+  }
   float r[8];
   if constexpr (sizeof(TX) == 4) {
     union { lt_u32x4 u[2]; float f[8]; } t;
