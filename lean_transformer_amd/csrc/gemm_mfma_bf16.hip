@@ -1,8 +1,13 @@
-// Tiled bf16 GEMM for gfx950 matrix cores (v_mfma_f32_32x32x16_bf16, fp32 accumulation) with the FFN epilogues fused.
+// Tiled bf16 GEMMs for gfx950 matrix cores (v_mfma_f32_32x32x16_bf16, fp32 accumulation) with the FFN epilogues fused.
+// Two kernels share the LDS layouts and the epilogues:
+//   gemm_bf16_dma_kernel  256 x 256 tile, operands copied global -> LDS without passing through registers; the kernel of
+//                         the dense projections (second half of this file)
+//   gemm_bf16_kernel      BM x BN tile, operands staged through registers; ragged reductions, the 128 x 128 tile of the
+//                         skinny low-rank GEMMs, and the block-sparse walks over 64 x 64 blocks
 //
-// Tile: BM x BN outputs per workgroup, 64 k per step, WM x WN wavefronts each owning a (BM/WM) x (BN/WN) sub-tile as
-// 32 x 32 MFMA blocks.  Operand tiles go global -> registers -> LDS (16-byte accesses) and are double-buffered in LDS:
-// while the matrix cores work on one stage the global loads of the next are in flight, with one barrier per k-step.
+// gemm_bf16_kernel.  Tile: BM x BN outputs per workgroup, 64 k per step, WM x WN wavefronts each owning a (BM/WM) x (BN/WN)
+// sub-tile as 32 x 32 MFMA blocks.  Operand tiles go global -> registers -> LDS (16-byte accesses) and are double-buffered
+// in LDS: while the matrix cores work on one stage the global loads of the next are in flight, with one barrier per k-step.
 //
 // Either operand may be stored k-major (k contiguous: activations x weights^T) or mn-major (k strided: transposed
 // activations in the weight-gradient GEMMs, weights in the input-gradient GEMMs):
@@ -471,8 +476,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
 //   mn-major  a ring of four [32 k][256] tiles, one k-step each; every row of a tile is 512 contiguous bytes in HBM.  The
 //             copy of k-step kt + 3 is issued during k-step kt.
 //   k-major   two [256][64 k] buffers, one block of two k-steps each, so that every row contributes a full 128-byte line
-//             to a copy (with 32 k per copy the L2 would see twice as many half-line requests).  The copy of block
-//             kt / 2 + 1 is issued during the even k-step kt.
+//             to a copy (with 32 k per copy the L2 would see twice as many half-line requests).  The two halves of the
+//             copy of block kt / 2 + 1 go out in slots around the even k-step kt (BlockSlots below).
 // Every LDS buffer is a separate array, so that copies into one provably do not alias reads of another.
 // Pipeline of k-step kt:
 //     matrix instructions on the first 16 k (fragments already in registers)
@@ -480,14 +485,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
 //     wait until this wavefront's copies of k-step kt + 1 have landed and its LDS reads are done; workgroup barrier
 //     matrix instructions on the second 16 k
 //         interleaved with: LDS reads of the first 16 k of k-step kt + 1
-// so no LDS read latency is exposed after the barrier and copies have 1.5 (k-major) to 2.5 (mn-major) k-steps to land.
+// so no LDS read latency is exposed after the barrier and copies have 1 to 2.5 k-steps to land.  The epilogue stages the
+// accumulators through LDS one 32-row strip at a time; whole tiles in the usual configurations take straight-line strips.
 // =====================================================================================================================
 __device__ const u32x4 lt_zero_chunk = {0u, 0u, 0u, 0u};  // source of the lanes past the end of a ragged reduction
 
 constexpr int DK = 32;  // k per step of the copy-based kernel
 
-// scheduling hint for one half k-step: READS LDS reads and COPIES global->LDS copies spread evenly over MFMAS matrix
-// instructions (packing the reads into the first half of the matrix instructions measured slower)
+// scheduling hint for one half k-step: READS LDS reads over the first READ_SPAN of MFMAS matrix instructions and COPIES
+// global->LDS copies evenly over all of them (packing the reads into the first quarter measured slower)
 template <int READS, int COPIES, int MFMAS, int READ_SPAN, int G = 0> struct SchedInterleave3 {
   static __device__ __forceinline__ void run() {
     // the LDS reads go out over the first SPAN matrix instructions, the copies over all of them
