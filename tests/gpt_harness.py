@@ -74,12 +74,19 @@ def attention_core(query, key, value, mask, cos, sin, num_heads: int):
 
 
 class Attention(nn.Module):
-    def __init__(self, cfg: GPTConfig):
+    def __init__(self, cfg: GPTConfig, linear_impl: str = "torch"):
+        """linear_impl: "torch" (nn.Linear) or "hip" (lean_transformer_amd.GeneralizedLinear on the HIP kernels, the layer
+        the reference builds for its attention projections: lean_transformer/transformer.py:48-61, config.py:172-182)"""
         super().__init__()
         self.cfg = cfg
         self.pre_layer_norm = nn.LayerNorm(cfg.hidden_size, eps=cfg.layer_norm_eps)
-        self.qkv_proj = nn.Linear(cfg.hidden_size, 3 * cfg.hidden_size)
-        self.out_proj = nn.Linear(cfg.hidden_size, cfg.hidden_size)
+        if linear_impl == "hip":
+            import lean_transformer_amd as lt
+            self.qkv_proj = lt.GeneralizedLinear(lt.GeneralizedMatrix(cfg.hidden_size, 3 * cfg.hidden_size), 0, True)
+            self.out_proj = lt.GeneralizedLinear(lt.GeneralizedMatrix(cfg.hidden_size, cfg.hidden_size), 0, True)
+        else:
+            self.qkv_proj = nn.Linear(cfg.hidden_size, 3 * cfg.hidden_size)
+            self.out_proj = nn.Linear(cfg.hidden_size, cfg.hidden_size)
 
     def forward(self, x, mask, cos, sin):
         qkv = self.qkv_proj(self.pre_layer_norm(x))
@@ -129,15 +136,16 @@ def _oracle_ffn_bf16(x: torch.Tensor, p: "offn.FFNParams") -> torch.Tensor:
 
 
 class MiniLeanGPT(nn.Module):
-    def __init__(self, cfg: GPTConfig, ffn_impl: str):
-        """ffn_impl: "hip" (lean_transformer_amd.LeanFFN, GPU only) or "oracle" (stock PyTorch, any device)"""
+    def __init__(self, cfg: GPTConfig, ffn_impl: str, linear_impl: str = "torch"):
+        """ffn_impl: "hip" (lean_transformer_amd.LeanFFN, GPU only) or "oracle" (stock PyTorch, any device);
+        linear_impl: what the attention projections are, "torch" or "hip" (see Attention)"""
         super().__init__()
         self.cfg = cfg
         E, H = cfg.embedding_size, cfg.hidden_size
         self.word_embeddings = nn.Embedding(cfg.vocab_size, E, padding_idx=cfg.pad_token_id)
         self.embedding_layer_norm = nn.LayerNorm(E, eps=cfg.layer_norm_eps)
         self.embedding_hidden_mapping = nn.Linear(E, H) if E != H else None
-        self.attentions = nn.ModuleList([Attention(cfg) for _ in range(cfg.num_layers)])
+        self.attentions = nn.ModuleList([Attention(cfg, linear_impl) for _ in range(cfg.num_layers)])
         if ffn_impl == "hip":
             import lean_transformer_amd as lt
             make = lambda: lt.LeanFFN(H, cfg.intermediate_size, gated=cfg.gated, layer_norm_eps=cfg.layer_norm_eps)
@@ -160,7 +168,7 @@ class MiniLeanGPT(nn.Module):
         gen = torch.Generator().manual_seed(seed)
         std = self.cfg.initializer_range
         for module in self.modules():
-            if isinstance(module, (nn.Linear, nn.Embedding)):
+            if isinstance(module, (nn.Linear, nn.Embedding)) or type(module).__name__ == "GeneralizedLinear":
                 module.weight.copy_(torch.randn(module.weight.shape, generator=gen) * std)
                 if getattr(module, "bias", None) is not None:
                     module.bias.zero_()
@@ -198,7 +206,15 @@ class MiniLeanGPT(nn.Module):
         return loss, logits
 
 
+def canonical_name(name: str) -> str:
+    """parameter name with the generalized linear layer's `matrix.` level removed (qkv_proj.matrix.weight -> qkv_proj.weight)"""
+    return name.replace(".matrix.weight", ".weight")
+
+
 def copy_parameters(src: MiniLeanGPT, dst: MiniLeanGPT):
-    """the two FFN implementations share parameter names, so the state dict carries over"""
-    missing, unexpected = dst.load_state_dict(src.state_dict(), strict=False)
-    assert not missing and not unexpected, (missing, unexpected)
+    """the implementations share parameter names up to the `matrix.` level of a generalized linear layer"""
+    source = {canonical_name(k): v for k, v in src.state_dict().items()}
+    with torch.no_grad():
+        for name, tensor in dst.state_dict().items():
+            tensor.copy_(source.pop(canonical_name(name)))
+    assert not source, sorted(source)

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from conftest import assert_close, cosine, rel_err
-from gpt_harness import GPTConfig, MiniLeanGPT, copy_parameters
+from gpt_harness import GPTConfig, MiniLeanGPT, canonical_name, copy_parameters
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -18,11 +18,11 @@ def _train_step(model, ids, autocast: bool):
     with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
         loss, _ = model(ids, labels=ids)
     loss.backward()
-    return loss.detach(), {name: p.grad.detach() for name, p in model.named_parameters()}
+    return loss.detach(), {canonical_name(name): p.grad.detach() for name, p in model.named_parameters()}
 
 
-def _pair(cfg):
-    hip, ref = MiniLeanGPT(cfg, "hip").to(DEV), MiniLeanGPT(cfg, "oracle").to(DEV)
+def _pair(cfg, linear_impl="torch"):
+    hip, ref = MiniLeanGPT(cfg, "hip", linear_impl).to(DEV), MiniLeanGPT(cfg, "oracle").to(DEV)
     copy_parameters(hip, ref)
     return hip, ref
 
@@ -38,6 +38,26 @@ def test_small_model_fp32():
     assert grads.keys() == grads_ref.keys()
     for name in grads:
         assert_close(grads[name], grads_ref[name], torch.float32, name)
+
+
+@pytest.mark.parametrize("autocast", [False, True])
+def test_small_model_attention_projections_on_the_hip_linear_layer(autocast):
+    """the attention's qkv and output projections as GeneralizedLinear on the HIP kernels too (the layer type the reference
+    builds there), FFN on the HIP kernels: loss and every gradient against the all-stock model"""
+    cfg = GPTConfig(vocab_size=1000, embedding_size=192, hidden_size=256, num_layers=2, num_heads=4,
+                    intermediate_size=512, layer_norm_eps=1e-5)
+    hip, ref = _pair(cfg, linear_impl="hip")
+    ids = torch.randint(0, cfg.vocab_size, (2, 128), generator=torch.Generator().manual_seed(1)).to(DEV)
+    loss, grads = _train_step(hip, ids, autocast=autocast)
+    loss_ref, grads_ref = _train_step(ref, ids, autocast=autocast)
+    assert abs(loss.item() - loss_ref.item()) <= (1e-3 if autocast else 1e-5) * abs(loss_ref.item())
+    assert grads.keys() == grads_ref.keys()
+    for name in grads:
+        if autocast:
+            err, cos = rel_err(grads[name], grads_ref[name]), cosine(grads[name], grads_ref[name])
+            assert err <= 5e-2 and cos >= 0.999, f"{name}: max relative error {err:.3e}, cosine {cos:.6f}"
+        else:
+            assert_close(grads[name], grads_ref[name], torch.float32, name)
 
 
 def test_config5_bf16_train_step():
