@@ -529,9 +529,11 @@ template <bool KM> struct DmaOperand {
   int64_t unit_bytes;
   int seg;
 
-  // row0: first row / column of the tile.  k-major only: rows are clamped below row_limit when row_limit > 0 (ragged M),
-  // and with pair_rows > 0 tile row r maps to the gated up-projection's weight rows (gate half, then linear half at
-  // + pair_rows), 64 of each per 128-row wavefront sub-tile.
+  // row0: first row / column of the tile; the operand has row_limit of them.  A tile that sticks out past row_limit copies
+  // the last row (k-major) or the last 8 columns (mn-major; row_limit is a multiple of 8) again in place of what is not
+  // there: those only feed result rows / columns that the epilogue does not write.  k-major with pair_rows > 0: tile row r
+  // maps to the gated up-projection's weight rows (gate half, then linear half at + pair_rows), 64 of each per 128-row
+  // wavefront sub-tile.
   __device__ __forceinline__ void setup(const GemmOperand& op, int s, int64_t row0, int64_t row_limit, int64_t pair_rows,
                                         int wave, int lane) {
     seg = s;
@@ -542,14 +544,15 @@ template <bool KM> struct DmaOperand {
       const int q = (wave * LOADS + j) * 64 + lane;  // 16-byte slot of the LDS buffer this lane fills
       if constexpr (KM) {
         const int row = q >> 3, c = (q & 7) ^ swz_km(row);
-        int64_t g = row;
-        if (row_limit > 0) g = min(row0 + row, row_limit - 1) - row0;
-        if (pair_rows > 0) g = ((row & 127) >> 6) * pair_rows + (row >> 7) * 64 + (row & 63);
+        const int local = pair_rows > 0 ? (row >> 7) * 64 + (row & 63) : row;
+        int64_t g = min(row0 + local, row_limit - 1) - row0;
+        if (pair_rows > 0) g += ((row & 127) >> 6) * pair_rows;
         off[j] = (uint32_t)((g * ld + c * 8) * 2);
         krow[j] = 0;
       } else {
         const int kr = q >> 5, c = (q & 31) ^ swz_mn(kr);
-        off[j] = (uint32_t)((kr * ld + c * 8) * 2);
+        const int64_t col = min(row0 + c * 8, row_limit - 8) - row0;
+        off[j] = (uint32_t)((kr * ld + col) * 2);
         krow[j] = kr;
       }
     }
@@ -661,8 +664,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   for (int j = 0; j < FN; j++) {
     bias0[j] = 0.f;
     if (p.epi.bias) {
-      const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) + n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31)
-                                : n0 + wn * WTN + j * 32 + (lane & 31);
+      // columns past N (a tile that sticks out) take the last column's bias and are never written
+      const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) +
+                                      min(n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31), p.N - 1)
+                                : min(n0 + wn * WTN + j * 32 + (lane & 31), p.N - 1);
       bias0[j] = p.epi.bias[col];
     }
   }
@@ -715,8 +720,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   };
   DmaOperand<A_KM> ca;
   DmaOperand<B_KM> cb;
-  auto setup_a = [&](int seg) { ca.setup(p.A[seg], seg, m0, A_KM ? p.M : 0, 0, wave, lane); };
-  auto setup_b = [&](int seg) { cb.setup(p.B[seg], seg, n0, 0, (B_KM && gated) ? p.N : 0, wave, lane); };
+  auto setup_a = [&](int seg) { ca.setup(p.A[seg], seg, m0, p.M, 0, wave, lane); };
+  auto setup_b = [&](int seg) { cb.setup(p.B[seg], seg, n0, p.N, (B_KM && gated) ? p.N : 0, wave, lane); };
   setup_a(0);
   setup_b(0);
   // copies of the unit that holds k-step t (a block for k-major operands) into the buffer of position I
@@ -960,26 +965,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
           vg[e] = sg[e];
           vl[e] = sl[e];
         }
-        if (m < p.M) epi_act_fwd_gated8(epi, m, n0 + wn * (WTN / 2) + c, vg, vl);
+        const int64_t n = n0 + wn * (WTN / 2) + c;
+        if (m < p.M && n < p.N) epi_act_fwd_gated8(epi, m, n, vg, vl);
       }
     } else {
       constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
       const int c = (lane % LANES_PER_ROW) * 8;
       const int64_t n = n0 + wn * WTN + c;
+      const bool in_n = n < p.N;  // N is a multiple of 8: the lane's 8 columns are all inside or all outside
       const int64_t mlane = mrow0 + lane / LANES_PER_ROW;  // this lane's row in iteration 0
       // global reads of the epilogue run two iterations ahead of their use
-      EpiLoad l0 = epi_load8<KIND, TX>(epi, mlane, n, mlane < p.M);
-      EpiLoad l1 = epi_load8<KIND, TX>(epi, mlane + ROWS_PER_IT, n, mlane + ROWS_PER_IT < p.M);
+      EpiLoad l0 = epi_load8<KIND, TX>(epi, mlane, n, in_n && mlane < p.M);
+      EpiLoad l1 = epi_load8<KIND, TX>(epi, mlane + ROWS_PER_IT, n, in_n && mlane + ROWS_PER_IT < p.M);
       for (int it = 0; it < NIT; it++) {
         const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
         const int64_t m = mrow0 + row;
         const int64_t m2 = m + 2 * ROWS_PER_IT;
-        const EpiLoad l2 = epi_load8<KIND, TX>(epi, m2, n, it + 2 < NIT && m2 < p.M);
+        const EpiLoad l2 = epi_load8<KIND, TX>(epi, m2, n, in_n && it + 2 < NIT && m2 < p.M);
         float v[8];
         const float* sv = staged(row, c);
 #pragma unroll
         for (int e = 0; e < 8; e++) v[e] = sv[e];
-        if (m < p.M) {
+        if (in_n && m < p.M) {
           if constexpr (KIND == EPI_STORE) epi_store8(epi, m, n, v);
           else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(epi, m, n, v);
           else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(epi, m, n, v, l0, colsum);
@@ -1019,7 +1026,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     __builtin_amdgcn_wave_barrier();
   };
   // The other kinds, same idea: whole tile in range, tanh GELU, no dropout, residual present.
-  const bool whole_tile = m0 + BM <= p.M;
+  const bool whole_tile = m0 + BM <= p.M && n0 + (gated ? BN / 2 : BN) <= p.N;
   auto act_fwd_strip = [&](auto I, auto G) {
     constexpr int i = decltype(I)::value;
     constexpr bool GATED = decltype(G)::value;
@@ -1114,7 +1121,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
         colsum[e] += __shfl_xor(colsum[e], 16);
         colsum[e] += __shfl_xor(colsum[e], 32);
       }
-      if (lane < 16) {
+      if (lane < 16 && n0 + wn * WTN + lane * 8 < p.N) {
         float* dst = epi.colsum + ((m0 + wm * WTM) / 128) * epi.ld_pre + n0 + wn * WTN + lane * 8;
         float lo[8], hi[8];
 #pragma unroll
@@ -1137,7 +1144,7 @@ int launch_dma(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
   else if (p.krot == 15) p.krot = 0;
   const bool gated = KIND == EPI_ACT_FWD && p.epi.gated;
   const int tiles_m = (int)((p.M + 255) / 256);
-  const int tiles_n = (int)(p.N / (gated ? 128 : 256));
+  const int tiles_n = (int)((p.N + (gated ? 127 : 255)) / (gated ? 128 : 256));
   bool k_tail = false;
   for (int s = 0; s < p.nseg; s++) k_tail = k_tail || (p.K[s] % DK != 0);
   dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(p.ksplit > 1 ? p.ksplit : 1)), block(256);
@@ -1246,11 +1253,15 @@ bool lt_gemm_mfma_supported(const GemmProblem& p, int kind) {
   constexpr int BM = 256, BN = 256;
   const bool gated = kind == EPI_ACT_FWD && p.epi.gated;
   if (p.M <= 0 || p.N <= 0) return false;
-  if (p.N % (gated ? BN / 2 : BN) != 0) return false;
+  const int64_t tile_n = gated ? BN / 2 : BN;
   const bool a_km = p.A[0].kmajor, b_km = p.B[0].kmajor;
   if (!a_km && b_km) return false;
-  if (!a_km && p.M % BM != 0) return false;  // mn-major A has no row clamp
-  if ((int64_t)((p.M + BM - 1) / BM) * (p.N / (gated ? BN / 2 : BN)) > 0x7fffffff) return false;
+  // Tiles that stick out past N (and past M for an mn-major A) are the copy-based kernel's: it copies the last row or the
+  // last 8 columns again and its epilogue skips what is outside, 8 columns at a time.
+  if (p.N % tile_n != 0 || (!a_km && p.M % BM != 0)) {
+    if (p.N % 8 != 0 || (!a_km && p.M % 8 != 0) || !dma_selected(p, kind, LT_BF16)) return false;
+  }
+  if ((int64_t)((p.M + BM - 1) / BM) * ((p.N + tile_n - 1) / tile_n) > 0x7fffffff) return false;
   // the epilogue moves 8 columns at a time
   const EpiParams& e = p.epi;
   if (e.bias && !lt_aligned(e.bias, 16)) return false;
@@ -1383,7 +1394,7 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
       LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
       return lt_splitk_reduce((const float*)workspace, slices, p.M * p.N, p.M * p.N, (int)p.N, e.bias, e.out_dtype, e.out, stream);
     }
-    if (((p.M + 255) / 256) * (p.N / 256) >= 64 || slices == 1) ok = false;
+    if (((p.M + 255) / 256) * ((p.N + 255) / 256) >= 64 || slices == 1) ok = false;
   }
   if (!ok) {
     // any-shape kernel: split the reduction when the tiles alone leave most workgroup slots empty

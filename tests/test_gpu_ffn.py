@@ -236,11 +236,18 @@ def test_ffn_bf16_one_row_past_a_tile(tokens):
     _compare(ffn, x, dy, torch.bfloat16)
 
 
-@pytest.mark.parametrize("hidden,inter", [(192, 320), (264, 520)])
-def test_ffn_bf16_sizes_off_the_tile_grid(hidden, inter):
-    """bf16 weights with hidden / intermediate sizes the 256-wide tiles do not divide: the any-shape kernel on bf16 operands"""
+@pytest.mark.parametrize("hidden,inter", [(192, 320), (264, 520), (320, 704)])
+@pytest.mark.parametrize("gated", [True, False])
+def test_ffn_bf16_sizes_off_the_tile_grid(hidden, inter, gated):
+    """bf16 weights with hidden / intermediate sizes the 256-wide tiles do not divide.  Multiples of 64: the tiled kernels
+    with tiles that stick out past the last column (and past the last row of the weight gradients); (264, 520): the
+    any-shape kernel on bf16 operands"""
     torch.manual_seed(hidden)
-    ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5).to(DEV).to(torch.bfloat16)
+    ffn = lt.LeanFFN(hidden, inter, gated=gated, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.i2h_proj.bias.normal_(std=0.1)
+        ffn.h2o_proj.bias.normal_(std=0.1)
+    ffn = ffn.to(DEV).to(torch.bfloat16)
     x, dy = torch.randn(300, hidden), torch.randn(300, hidden)
     _compare(ffn, x, dy, torch.bfloat16)
 

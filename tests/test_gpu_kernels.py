@@ -75,6 +75,42 @@ def test_gemm_tiled_bf16_ragged_rows_and_reduction():
     assert rel_err(_gemm(a, b, False, False, 512, 256, 1000, torch.float32, False), ref) <= 1e-5
 
 
+def _kernel_tags(fn):
+    """runs fn with the library's kernel timing on and returns the tags of the kernels it launched"""
+    lib = nat.lib()
+    lib.lt_profile_reset()
+    lib.lt_profile_enable(1)
+    try:
+        out = fn()
+        torch.cuda.synchronize()
+    finally:
+        lib.lt_profile_enable(0)
+    tags = {entry[0] for entry in nat.profile_read()}
+    lib.lt_profile_reset()
+    return out, tags
+
+
+@pytest.mark.parametrize("a_kmajor,b_kmajor,tag", [(True, True, "gemm_bf16_nt_store"), (True, False, "gemm_bf16_nn_store"),
+                                                   (False, False, "gemm_bf16_tn_store")])
+@pytest.mark.parametrize("m,n,k", [(512, 320, 128), (256, 8, 64), (328, 200, 192), (1600, 1608, 320), (264, 776, 448)])
+@pytest.mark.parametrize("c_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_tiled_bf16_tiles_past_the_edge(a_kmajor, b_kmajor, tag, m, n, k, c_dtype):
+    """N (and, for an mn-major A, M) a multiple of 8 but not of the 256-wide tile: the tiled kernel still takes the problem,
+    re-reads the last row / last 8 columns for the part of the tile that sticks out and writes nothing there"""
+    a, b, ref = _operands(m, n, k, a_kmajor, b_kmajor, torch.bfloat16, seed=m + 2 * n + 3 * k)
+    flat = torch.full((m * n + 4096,), 7.0, dtype=c_dtype, device=DEV)  # the result, then a guard nothing may write
+    c = flat[:m * n].view(m, n)
+    _, tags = _kernel_tags(lambda: nat.check(
+        nat.lib().lt_gemm(nat.dtype_code(a.dtype), m, n, k, nat.ptr(a), int(a_kmajor), nat.ptr(b), int(b_kmajor),
+                          nat.dtype_code(c_dtype), nat.ptr(c), 0, nat.current_stream(c.device)), "lt_gemm"))
+    assert tag in tags, tags
+    assert bool((flat[m * n:] == 7.0).all())
+    if c_dtype == torch.float32:
+        assert rel_err(c, ref) <= 1e-5
+    else:
+        assert_close(c, ref.float(), torch.bfloat16, "c")
+
+
 @pytest.mark.parametrize("tokens,hidden", [(37, 32), (64, 768), (9, 4096), (3, 10), (5, 8192), (2, 8200)])
 @pytest.mark.parametrize("x_dtype,y_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
                                              (torch.bfloat16, torch.bfloat16)])
