@@ -112,6 +112,7 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
     p.K[0] = in;
     p.A[0] = operand(x, in, true);
     p.B[0] = operand(lin.weight, in, true);
+    if (kind == EPI_OUT && r == 0) return lt_launch_gemm_out(p, dtype, io_dtype, skinny_ws, skinny_bytes, stream);
     return lt_launch_gemm(p, kind, dtype, io_dtype, stream);
   }
   LT_REQUIRE(!gated, LT_ERR_UNSUPPORTED, "internal: gated epilogue on a block-sparse projection");
@@ -263,6 +264,11 @@ void plan_forward(const lt_ffn_desc& d, Bump& ws, FwdScratch& s) {
   s.hid = ws.take((size_t)d.tokens * d.intermediate * e);
   const int r = d.i2h.lowrank > d.h2o.lowrank ? d.i2h.lowrank : d.h2o.lowrank;
   s.skinny_bytes = r > 0 ? lt_gemm_skinny_workspace(d.tokens, r) : 0;
+  // dense down-projection of a short batch: room to split its reduction, no more than the saved pre-activation takes
+  if (d.compute_dtype == LT_BF16 && d.h2o.block == 0 && d.h2o.lowrank == 0 && !d.post_ln_weight) {
+    const size_t cap = (size_t)d.tokens * (d.gated ? 2 : 1) * d.intermediate * e;
+    s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_out_splitk_workspace(d.tokens, d.hidden, d.intermediate, cap));
+  }
   s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 

@@ -1440,6 +1440,63 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
   return lt_splitk_reduce((const float*)workspace, slices, p.M * p.N, p.M * p.N, (int)p.N, e.bias, e.out_dtype, e.out, stream);
 }
 
+namespace {
+// sum of the split-k slices of an [M, N] result, 8 columns per thread, through the EPI_OUT epilogue (bias, dropout, residual)
+template <typename TX>
+__global__ __launch_bounds__(256) void splitk_reduce_out_kernel(const float* __restrict__ partial, int slices, int64_t stride,
+                                                                 int64_t M, int64_t N, EpiParams e) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i >= M * N) return;
+  float v[8];
+  load8(partial + i, v);
+  for (int s = 1; s < slices; s++) {
+    float w[8];
+    load8(partial + (int64_t)s * stride + i, w);
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] += w[k];
+  }
+  epi_out8<TX>(e, i / N, i % N, v);
+}
+}  // namespace
+
+size_t lt_gemm_out_splitk_workspace(int64_t M, int64_t N, int64_t K, size_t cap_bytes) {
+  const size_t full = lt_gemm_splitk_workspace(M, N, K);
+  const size_t slice = (size_t)M * (size_t)N * sizeof(float);
+  if (full == 0 || cap_bytes < 2 * slice) return 0;
+  return std::min(full, lt_align_up(cap_bytes / slice * slice, 256));
+}
+
+int lt_launch_gemm_out(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
+                       hipStream_t stream) {
+  const EpiParams& e = p.epi;
+  if (dtype == LT_BF16 && p.nseg == 1 && p.sp.mode == SPARSE_NONE && workspace && p.N % 8 == 0 && e.ldy % 8 == 0 &&
+      lt_aligned(e.y, 16) && (!e.x || lt_aligned(e.x, 16)) && (!e.bias || lt_aligned(e.bias, 16)) && g_mfma_variant != 1 &&
+      p.K[0] % 64 == 0) {
+    GemmProblem q = p;
+    q.epi = EpiParams{};
+    q.epi.out = workspace;
+    q.epi.ldo = p.N;
+    q.epi.out_dtype = LT_F32;
+    const size_t slice = (size_t)p.M * (size_t)p.N * sizeof(float);
+    const int slices = (int)std::min<size_t>((size_t)splitk_slices(p.M, p.N, p.K[0]), workspace_bytes / slice);
+    if (slices > 1 && lt_gemm_mfma_supported(q, EPI_STORE) && dma_offsets_fit(q, EPI_STORE)) {
+      q.ksplit = slices;
+      q.split_stride = p.M * p.N;
+      LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+      LtProfileScope scope("splitk_reduce_out", 0.0,
+                           (double)p.M * p.N * (4.0 * slices + (e.x ? 2 : 1) * lt_dtype_size(io_dtype)), stream);
+      const dim3 grid((unsigned)((p.M * p.N / 8 + 255) / 256)), block(256);
+      if (io_dtype == LT_BF16)
+        hipLaunchKernelGGL((splitk_reduce_out_kernel<bf16>), grid, block, 0, stream, (const float*)workspace, slices, p.M * p.N, p.M, p.N, e);
+      else
+        hipLaunchKernelGGL((splitk_reduce_out_kernel<float>), grid, block, 0, stream, (const float*)workspace, slices, p.M * p.N, p.M, p.N, e);
+      LT_LAUNCH_CHECK();
+      return LT_OK;
+    }
+  }
+  return lt_launch_gemm(p, EPI_OUT, dtype, io_dtype, stream);
+}
+
 // block-sparse walk on the matrix cores: 64 x 64 blocks, bf16, 16-byte aligned operands
 bool lt_sparse_mfma_supported(const GemmProblem& p, int kind) {
   const SparseWalk& sp = p.sp;

@@ -471,6 +471,13 @@ int lt_gemm_colsum_rows(const GemmProblem& p, int dtype, int io_dtype);
 int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream);
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                           hipStream_t stream);
+// EPI_OUT problems with few output tiles and a long reduction (the down-projection of a short batch): the reduction split
+// over workgroups into fp32 partial sums in `workspace`, then one pass that sums them through the same epilogue.  Takes as
+// many slices as the workspace holds; falls back to lt_launch_gemm when the shape does not fit or one slice is enough.
+// lt_gemm_out_splitk_workspace: bytes worth having for an [M, N] result, at most cap_bytes (0: no split would be taken).
+size_t lt_gemm_out_splitk_workspace(int64_t M, int64_t N, int64_t K, size_t cap_bytes);
+int lt_launch_gemm_out(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
+                       hipStream_t stream);
 // out[i] = sum_s partial[s * stride + i] (+ bias[i % cols]) for i < count, cast to out_dtype
 int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t count, int cols, const float* bias,
                      int out_dtype, void* out, hipStream_t stream);

@@ -153,11 +153,13 @@ def test_ffn_dropout_behaviour():
 
 @pytest.mark.parametrize("post_ln", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_ffn_dropout_mask_parity(post_ln, dtype):
+@pytest.mark.parametrize("inter", [512, 2048])
+def test_ffn_dropout_mask_parity(post_ln, dtype, inter):
     """the mask is never stored: forward epilogue and backward replay evaluate the same Philox stream.  Hand the oracle the
-    mask of that stream and compare everything; seeding the generator reproduces the run."""
+    mask of that stream and compare everything; seeding the generator reproduces the run.  With intermediate size 2048 the
+    bf16 down-projection splits its reduction and the pass that sums the slices draws the mask."""
     torch.manual_seed(3)
-    hidden, inter, tokens = 256, 512, 300
+    hidden, tokens = 256, 300
     ffn = lt.LeanFFN(hidden, inter, dropout=0.1, post_layer_norm=post_ln, layer_norm_eps=1e-5)
     with torch.no_grad():
         ffn.i2h_proj.weight.normal_(std=0.05)
@@ -183,6 +185,33 @@ def test_ffn_dropout_mask_parity(post_ln, dtype):
     torch.cuda.manual_seed(77)
     y2, dx2, _ = _run_module(ffn, x.to(DEV), dy.to(DEV))
     assert torch.equal(y, y2) and torch.equal(dx, dx2)
+
+
+@pytest.mark.parametrize("io_dtype", [torch.float32, torch.bfloat16])
+def test_short_batch_down_projection_splits_its_reduction(io_dtype):
+    """few tokens, long intermediate size: the down-projection has too few tiles for the chip, so its reduction is split and a
+    second pass sums the slices through the bias / residual epilogue.  Checks that this path is the one that ran."""
+    from lean_transformer_amd import _native as nat
+
+    torch.manual_seed(11)
+    ffn = lt.LeanFFN(512, 4096, gated=True, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.h2o_proj.bias.normal_(std=0.1)
+    ffn = ffn.to(DEV).to(torch.bfloat16)
+    x, dy = torch.randn(200, 512).to(io_dtype), torch.randn(200, 512).to(io_dtype)
+    lib = nat.lib()
+    lib.lt_profile_reset()
+    lib.lt_profile_enable(1)
+    try:
+        with torch.no_grad():
+            ffn(x.to(DEV))
+        torch.cuda.synchronize()
+    finally:
+        lib.lt_profile_enable(0)
+    tags = {entry[0] for entry in nat.profile_read()}
+    lib.lt_profile_reset()
+    assert "splitk_reduce_out" in tags, tags
+    _compare(ffn, x, dy, torch.bfloat16)
 
 
 def _c1():
