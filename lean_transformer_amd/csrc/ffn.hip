@@ -265,7 +265,7 @@ void plan_forward(const lt_ffn_desc& d, Bump& ws, FwdScratch& s) {
   const int r = d.i2h.lowrank > d.h2o.lowrank ? d.i2h.lowrank : d.h2o.lowrank;
   s.skinny_bytes = r > 0 ? lt_gemm_skinny_workspace(d.tokens, r) : 0;
   // dense down-projection of a short batch: room to split its reduction, no more than the saved pre-activation takes
-  if (d.compute_dtype == LT_BF16 && d.h2o.block == 0 && d.h2o.lowrank == 0 && !d.post_ln_weight) {
+  if (d.h2o.block == 0 && d.h2o.lowrank == 0 && !d.post_ln_weight) {
     const size_t cap = (size_t)d.tokens * (d.gated ? 2 : 1) * d.intermediate * e;
     s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_out_splitk_workspace(d.tokens, d.hidden, d.intermediate, cap));
   }

@@ -1460,7 +1460,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_out_kernel(const float* __r
 }  // namespace
 
 size_t lt_gemm_out_splitk_workspace(int64_t M, int64_t N, int64_t K, size_t cap_bytes) {
-  const size_t full = lt_gemm_splitk_workspace(M, N, K);
+  const size_t full = std::max(lt_gemm_splitk_workspace(M, N, K), lt_gemm_generic_splitk_workspace(M, N, K));
   const size_t slice = (size_t)M * (size_t)N * sizeof(float);
   if (full == 0 || cap_bytes < 2 * slice) return 0;
   return std::min(full, lt_align_up(cap_bytes / slice * slice, 256));
@@ -1469,20 +1469,26 @@ size_t lt_gemm_out_splitk_workspace(int64_t M, int64_t N, int64_t K, size_t cap_
 int lt_launch_gemm_out(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                        hipStream_t stream) {
   const EpiParams& e = p.epi;
-  if (dtype == LT_BF16 && p.nseg == 1 && p.sp.mode == SPARSE_NONE && workspace && p.N % 8 == 0 && e.ldy % 8 == 0 &&
-      lt_aligned(e.y, 16) && (!e.x || lt_aligned(e.x, 16)) && (!e.bias || lt_aligned(e.bias, 16)) && g_mfma_variant != 1 &&
-      p.K[0] % 64 == 0) {
+  if (p.nseg == 1 && p.sp.mode == SPARSE_NONE && workspace && lt_aligned(workspace, 16) && p.M > 0 && p.N > 0 &&
+      p.N % 8 == 0 && e.ldy % 8 == 0 && lt_aligned(e.y, 16) && (!e.x || lt_aligned(e.x, 16)) &&
+      (!e.bias || lt_aligned(e.bias, 16))) {
     GemmProblem q = p;
     q.epi = EpiParams{};
     q.epi.out = workspace;
     q.epi.ldo = p.N;
     q.epi.out_dtype = LT_F32;
     const size_t slice = (size_t)p.M * (size_t)p.N * sizeof(float);
-    const int slices = (int)std::min<size_t>((size_t)splitk_slices(p.M, p.N, p.K[0]), workspace_bytes / slice);
-    if (slices > 1 && lt_gemm_mfma_supported(q, EPI_STORE) && dma_offsets_fit(q, EPI_STORE)) {
+    // the tiled kernel where it takes the problem (a k-major reduction splits in blocks of 64), else the any-shape kernel
+    const bool tiled = dtype == LT_BF16 && g_mfma_variant != 1 && p.K[0] % 64 == 0 && lt_gemm_mfma_supported(q, EPI_STORE) &&
+                       dma_offsets_fit(q, EPI_STORE);
+    const bool tiled_unsplit = dtype == LT_BF16 && lt_gemm_mfma_supported(p, EPI_OUT);
+    const int wanted = tiled ? splitk_slices(p.M, p.N, p.K[0]) : tiled_unsplit ? 1 : generic_splitk_slices(p.M, p.N, p.K[0]);
+    const int slices = (int)std::min<size_t>((size_t)wanted, workspace_bytes / slice);
+    if (slices > 1) {
       q.ksplit = slices;
       q.split_stride = p.M * p.N;
-      LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+      if (tiled) LT_TRY(lt_launch_gemm(q, EPI_STORE, dtype, io_dtype, stream));
+      else LT_TRY(lt_launch_gemm_generic(q, EPI_STORE, dtype, io_dtype, stream));
       LtProfileScope scope("splitk_reduce_out", 0.0,
                            (double)p.M * p.N * (4.0 * slices + (e.x ? 2 : 1) * lt_dtype_size(io_dtype)), stream);
       const dim3 grid((unsigned)((p.M * p.N / 8 + 255) / 256)), block(256);
