@@ -508,12 +508,13 @@ template <int READS, int COPIES, int MFMAS, int READ_SPAN, int G = 0> struct Sch
   }
 };
 
-// wait until at most N of this wavefront's copies are in flight and all its LDS reads have returned, then barrier.
+// wait until at most N of this wavefront's copies are in flight and (WAIT_LDS) all its LDS reads have returned, then barrier.
 // The wait is a real s_waitcnt instruction (not inline assembly) so that the compiler's own wait-count bookkeeping sees
 // that older copies have landed; the empty asm statements only keep it from moving LDS accesses across the barrier.
-template <int N> __device__ __forceinline__ void wait_copies_and_barrier() {
+template <int N, bool WAIT_LDS = true> __device__ __forceinline__ void wait_copies_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));  // vmcnt(N) expcnt(7: none) lgkmcnt(0)
+  // vmcnt(N) expcnt(7: none) lgkmcnt(0, or 15: none)
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | ((WAIT_LDS ? 0 : 15) << 8));
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -564,6 +565,19 @@ template <bool KM> struct DmaOperand {
   // J0, J1: range of this wavefront's copy instructions (a k-major block can go out in two halves)
   template <bool K_TAIL, int J0 = 0, int J1 = LOADS>
   __device__ __forceinline__ void issue(int u, bf16* dst, int wave, int64_t k_limit) const {
+    if constexpr (!(K_TAIL && !KM)) {
+      // Buffer form: wavefront-uniform descriptor of the unit + the lane's 32-bit offset.  No vector address arithmetic,
+      // and unlike the global form the compiler does not count it as a FLAT access, after which it turns every wait for
+      // LDS data into a wait for all of it.
+      const __amdgpu_buffer_rsrc_t rsrc =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base + u * unit_bytes), 0, -1, 0x00020000);
+#pragma unroll
+      for (int j = J0; j < J1; j++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + (wave * LOADS + j) * 512),
+                                                 16, (int)off[j], 0, 0, 0);
+      return;
+    }
+    // ragged reduction over mn-major operands: lanes past the end read a chunk of zeros instead
 #pragma unroll
     for (int j = J0; j < J1; j++) {
       const char* g = base + u * unit_bytes + off[j];
@@ -766,15 +780,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     constexpr int half = decltype(I)::value & 1;
     const bf16* ta = a_buf(I);
     const bf16* tb = b_buf(I);
+    // pair (A block i, B block i) after pair i - 1: the order in which the matrix instructions below first need them
+    static_assert(FM == FN, "reads alternate between the operands");
 #pragma unroll
     for (int i = 0; i < FM; i++) {
       if constexpr (A_KM) a[i] = frag_km(ta, wm * WTM + i * 32, kk, half);
       else a[i] = frag_mn(ta, wm * WTM + i * 32, kk);
+      if constexpr (B_KM) b[i] = frag_km(tb, wn * WTN + i * 32, kk, half);
+      else b[i] = frag_mn(tb, wn * WTN + i * 32, kk);
     }
+  };
+  // the 16 matrix instructions of a half-step, in the order in which their fragments arrive (pair 0 first, pair 3 last):
+  // the wait before the first one then covers two LDS reads, not all eight
+  auto mfma_half = [&](bf16x8 (&a)[FM], bf16x8 (&b)[FN]) {
+    constexpr int ORDER[16][2] = {{0, 0}, {1, 0}, {0, 1}, {1, 1}, {2, 0}, {2, 1}, {0, 2}, {1, 2},
+                                  {2, 2}, {3, 0}, {3, 1}, {3, 2}, {0, 3}, {1, 3}, {2, 3}, {3, 3}};
 #pragma unroll
-    for (int j = 0; j < FN; j++) {
-      if constexpr (B_KM) b[j] = frag_km(tb, wn * WTN + j * 32, kk, half);
-      else b[j] = frag_mn(tb, wn * WTN + j * 32, kk);
+    for (int q = 0; q < 16; q++) {
+      const int x = ORDER[q][0], y = ORDER[q][1];
+      acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y], 0, 0, 0);
     }
   };
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);
@@ -824,10 +848,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       if (STEADY || t + 2 < kt_total)
         copy_block_halves(steady, std::integral_constant<int, 1>{}, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
     }
-#pragma unroll
-    for (int x = 0; x < FM; x++)
-#pragma unroll
-      for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][x], bfr[0][y], acc[x][y], 0, 0, 0);
+    mfma_half(af[0], bfr[0]);
     constexpr int COPIES = (A_KM ? 0 : 4) + ((B_KM || B_SPLIT) ? 0 : 4) + ((i & 1) == 0 ? slot_copies(1) : 0);
     SchedInterleave3<FRAG_READS, COPIES, FM * FN, READ_SPAN>::run();
   };
@@ -835,7 +856,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
     constexpr int IN_FLIGHT = copies_in_flight(A_KM, B_KM, SA, SB, B_SPLIT, i & 1);
-    if constexpr (STEADY) wait_copies_and_barrier<IN_FLIGHT>();
+    // LDS reads in flight here are the second 16 k of k-step t (position i).  Copies issued before the next barrier that
+    // overwrite that buffer: mn-major copies of the next first half (the ring tile of k-step t), and after an odd k-step
+    // the slot-0 and slot-1 halves of a k-major block.  Without those the reads may stay in flight across the barrier.
+    constexpr bool READS_MUST_LAND = !A_KM || (!B_KM && !B_SPLIT) ||
+                                     (N_KM > 0 && (i & 1) == 1 && slot_copies(0) + slot_copies(1) > 0);
+    if constexpr (STEADY) wait_copies_and_barrier<IN_FLIGHT, READS_MUST_LAND>();
     else wait_copies_and_barrier<0>();
     if (STEADY || t + 1 < kt_total) load_frags(std::integral_constant<int, (i + 1) & 3>{}, 0, af[0], bfr[0]);
     // the barrier above freed the buffers of k-step t - 1 and, on odd t, the k-major buffer of k-steps t - 1, t
@@ -850,10 +876,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       if (STEADY || t + 2 < kt_total)
         copy_block_halves(steady, std::integral_constant<int, 2>{}, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
     }
-#pragma unroll
-    for (int x = 0; x < FM; x++)
-#pragma unroll
-      for (int y = 0; y < FN; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][x], bfr[1][y], acc[x][y], 0, 0, 0);
+    mfma_half(af[1], bfr[1]);
     constexpr int COPIES = (B_SPLIT ? 4 : 0) + (N_KM > 0 ? slot_copies((i & 1) ? 0 : 2) : 0);
     SchedInterleave3<FRAG_READS, COPIES, FM * FN, READ_SPAN>::run();
   };
