@@ -836,6 +836,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     return (A_KM ? 4 * ((SA.half[0] == slot) + (SA.half[1] == slot)) : 0) +
            (B_KM ? 4 * ((SB.half[0] == slot) + (SB.half[1] == slot)) : 0);
   };
+  // LDS reads in flight at the barrier of k-step t are the second 16 k of that k-step (position i).  Copies issued before
+  // the next barrier that overwrite that buffer: mn-major copies of the next first half (the ring tile of k-step t), and
+  // after an odd k-step the slot-0 and slot-1 halves of a k-major block.  Without those the reads may stay in flight
+  // across the barrier.
+  constexpr bool MN_FIRST_HALF = !A_KM || (!B_KM && !B_SPLIT);
+  constexpr bool KM_EARLY_SLOTS = (A_KM && (SA.half[0] < 2 || SA.half[1] < 2)) || (B_KM && (SB.half[0] < 2 || SB.half[1] < 2));
   auto first_half = [&](auto steady, auto I, int t) {
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
@@ -856,11 +862,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     constexpr bool STEADY = decltype(steady)::value;
     constexpr int i = decltype(I)::value & 3;
     constexpr int IN_FLIGHT = copies_in_flight(A_KM, B_KM, SA, SB, B_SPLIT, i & 1);
-    // LDS reads in flight here are the second 16 k of k-step t (position i).  Copies issued before the next barrier that
-    // overwrite that buffer: mn-major copies of the next first half (the ring tile of k-step t), and after an odd k-step
-    // the slot-0 and slot-1 halves of a k-major block.  Without those the reads may stay in flight across the barrier.
-    constexpr bool READS_MUST_LAND = !A_KM || (!B_KM && !B_SPLIT) ||
-                                     (N_KM > 0 && (i & 1) == 1 && slot_copies(0) + slot_copies(1) > 0);
+    constexpr bool READS_MUST_LAND = MN_FIRST_HALF || ((i & 1) == 1 && KM_EARLY_SLOTS);
     if constexpr (STEADY) wait_copies_and_barrier<IN_FLIGHT, READS_MUST_LAND>();
     else wait_copies_and_barrier<0>();
     if (STEADY || t + 1 < kt_total) load_frags(std::integral_constant<int, (i + 1) & 3>{}, 0, af[0], bfr[0]);
