@@ -1403,7 +1403,10 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
             p.A[0].ld % 8 == 0 && p.B[0].ld % 8 == 0 && lt_aligned(p.A[0].ptr, 16) && lt_aligned(p.B[0].ptr, 16) &&
             e.ldo == p.N && lt_aligned(e.out, 16) && (!e.bias || lt_aligned(e.bias, 16));
   const int64_t tiles = ((p.M + 127) / 128) * (p.N / 128);
-  if (dtype == LT_BF16 && p.sp.mode == SPARSE_NONE && lt_gemm_mfma_supported(p, EPI_STORE)) {
+  // a result only 128 wide (or, for an mn-major A, 128 tall) would leave half of every 256 x 256 tile empty: the 128 x 128
+  // tile below takes it when it can
+  const bool half_tiles = ok && (p.N == 128 || (!a_km && p.M == 128));
+  if (!half_tiles && dtype == LT_BF16 && p.sp.mode == SPARSE_NONE && lt_gemm_mfma_supported(p, EPI_STORE)) {
     // 256 x 256 tiles fit: the copy-based kernel, its reduction split when the tiles alone leave CUs idle
     const int slices = p.nseg == 1 ? splitk_slices(p.M, p.N, p.K[0]) : 1;
     const size_t need = (size_t)slices * (size_t)p.M * (size_t)p.N * sizeof(float);
