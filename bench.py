@@ -101,6 +101,38 @@ def cpu_baseline(torch, hidden, inter, std, sample_tokens, iters):
     return sample_tokens / best, best
 
 
+def library_gemm_yardstick(torch, cfg, device, iters=10):
+    """torch.matmul (the vendor GEMM library) in bf16 on the six GEMM shapes of a dense step, each in the operand layout the
+    step has it in, with no epilogue work: what a plain library GEMM reaches on the same box in the same run.  Not part of
+    the product path; reported next to the library's own per-kernel figures."""
+    tokens, hidden, inter = cfg["batch"] * cfg["seq"], cfg["hidden"], cfg["inter"]
+    n1 = 2 * inter if cfg["gated"] else inter
+    # name: (M, N, K, layout); nt: A [M,K], B [N,K]; nn: A [M,K], B [K,N]; tn: A [K,M], B [K,N]
+    shapes = {"up": (tokens, n1, hidden, "nt"), "down": (tokens, hidden, inter, "nt"), "dh": (tokens, inter, hidden, "nn"),
+              "dW2": (hidden, inter, tokens, "tn"), "du": (tokens, hidden, n1, "nn"), "dW1": (n1, hidden, tokens, "tn")}
+    out, total_us, total_flops = {}, 0.0, 0.0
+    for name, (m, n, k, layout) in shapes.items():
+        a = torch.randn((k, m) if layout == "tn" else (m, k), device=device, dtype=torch.bfloat16)
+        b = torch.randn((n, k) if layout == "nt" else (k, n), device=device, dtype=torch.bfloat16)
+        fn = {"nt": lambda: a @ b.t(), "nn": lambda: a @ b, "tn": lambda: a.t() @ b}[layout]
+        for _ in range(3):
+            fn()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        us = start.elapsed_time(stop) / iters * 1e3
+        out[name] = {"m": m, "n": n, "k": k, "layout": layout, "avg_us": us, "tflops": 2.0 * m * n * k / us / 1e6}
+        total_us += us
+        total_flops += 2.0 * m * n * k
+        del a, b
+    out["all"] = {"avg_us": total_us / len(shapes), "tflops": total_flops / total_us / 1e6}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +141,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing (profiling runs)")
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS), help="benchmark configuration (default: the "
                     "headline config 3; the others are reported for reference)")
+    ap.add_argument("--yardstick", action="store_true", help="also time torch.matmul (vendor GEMM library, no epilogue) on "
+                    "the six GEMM shapes of the step, for comparison (dense configurations)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no collectives and every box has one GPU (use --gpus 1)")
@@ -213,6 +247,8 @@ def main():
             "value": value, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"oracle LeanFFNFunction (stock PyTorch fp32, reference save-set) on the first {sample} of {tokens} "
                       f"tokens of config 3, median of 3 fwd+bwd after 1 warm-up, {sec:.2f} s each"}
+    if args.yardstick and not cfg["sparse"] and cfg["dtype"] == "bf16":
+        result["library_gemm_yardstick"] = library_gemm_yardstick(torch, cfg, device)
     print(json.dumps(result))
 
 
