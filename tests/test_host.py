@@ -94,6 +94,37 @@ def test_generalized_linear_parameter_layout():
     assert a.weight is b.weight and a.adapter_first is not b.adapter_first
 
 
+def test_checkpoint_round_trip_in_the_reference_key_layout(tmp_path):
+    """A checkpoint written from the module holds exactly the keys the reference's module would write (nn.Linear:
+    ffn.py:51-52; GeneralizedLinear: blocksparse/linear.py:32-66, 109-123, layout and index tables as persistent buffers)
+    and loads back strictly, from a file read with weights_only=True, into a freshly constructed module."""
+    torch.manual_seed(0)
+
+    def sparse_ffn():
+        up = lt.GeneralizedLinear(lt.GeneralizedMatrix(32, 256, "pixelfly(16)", lowrank_dim=4), adapter_dim=2)
+        down = lt.GeneralizedLinear(lt.GeneralizedMatrix(128, 32, "pixelfly(16)", lowrank_dim=4), adapter_dim=2)
+        return lt.LeanFFN(32, 128, gated=True, i2h_proj=up, h2o_proj=down)
+
+    for make in (lambda: lt.LeanFFN(32, 128, gated=True, post_layer_norm=True), sparse_ffn):
+        src, dst = make(), make()
+        with torch.no_grad():
+            for t in src.parameters():
+                t.normal_()
+        path = tmp_path / "ffn.pth"
+        torch.save(src.state_dict(), path)
+        state = torch.load(path, weights_only=True)
+        assert list(state) == list(src.state_dict())
+        result = dst.load_state_dict(state, strict=True)
+        assert not result.missing_keys and not result.unexpected_keys
+        for key, value in src.state_dict().items():
+            assert torch.equal(dst.state_dict()[key], value) and dst.state_dict()[key].dtype == value.dtype, key
+    sparse = sparse_ffn().state_dict()
+    assert sparse["i2h_proj.matrix.layout"].dtype == torch.bool and tuple(sparse["i2h_proj.matrix.layout"].shape) == (16, 2)
+    assert sparse["i2h_proj.matrix.forward_indices"].dtype == torch.int32
+    assert sparse["i2h_proj.matrix.backward_indices"].dtype == torch.int64
+    assert tuple(sparse["i2h_proj.matrix.weight"].shape) == (32, 16, 16)  # native order [in_features, A, block]
+
+
 def test_activation_mapping():
     assert activation_kind(ACT2FN["gelu_fused"]) == "gelu_fused"
     assert activation_kind(ACT2FN["gelu_new"]) == "gelu_fused"
