@@ -183,6 +183,34 @@ def test_activation_forward_backward(act, gated, dtype):
     assert_close(dpre, dpre_ref.float(), dtype, "dpre")
 
 
+def test_tanh_gelu_saturates_cleanly_in_the_bf16_kernels():
+    """the bf16 kernels evaluate the tanh GELU through a sigmoid with fast exp2 / rcp: far in the tails (e^{-2u} over- or
+    underflowing) value and derivative must come out as the limits x / 0 and 1 / 0, never NaN or inf, and in between they
+    must follow the closed forms of the reference (utils.py:24-38)"""
+    from lean_transformer_amd.utils import ACT_KINDS
+    x = torch.tensor([-3.0e4, -1.0e3, -100.0, -30.0, -12.0, -6.0, -3.0, -1.0, -0.25, -1e-3, 0.0, 1e-3, 0.25, 1.0, 3.0, 6.0,
+                      12.0, 30.0, 100.0, 1.0e3, 3.0e4] + [0.0] * 11).view(4, 8)
+    tokens, inter = x.shape
+    pre = x.to(torch.bfloat16).to(DEV)
+    dh = torch.ones_like(pre)
+    hid, dpre = torch.empty_like(pre), torch.empty_like(pre)
+    lib = nat.lib()
+    nat.check(lib.lt_activation_forward(tokens, inter, 0, ACT_KINDS["gelu_fused"], nat.dtype_code(torch.bfloat16),
+                                        nat.ptr(pre), nat.ptr(hid), nat.current_stream(pre.device)), "lt_activation_forward")
+    nat.check(lib.lt_activation_backward(tokens, inter, 0, ACT_KINDS["gelu_fused"], nat.dtype_code(torch.bfloat16),
+                                         nat.ptr(pre), nat.ptr(dh), nat.ptr(dpre), nat.current_stream(pre.device)),
+              "lt_activation_backward")
+    xf = pre.float().cpu().double()
+    value = offn.gelu_fused(xf)
+    grad = offn.gelu_fused_grad(torch.ones_like(xf), xf)
+    hid, dpre = hid.float().cpu().double(), dpre.float().cpu().double()
+    assert torch.isfinite(hid).all() and torch.isfinite(dpre).all()
+    assert torch.allclose(hid, value, rtol=1e-2, atol=1e-6), (hid - value).abs().max()
+    assert torch.allclose(dpre, grad, rtol=1e-2, atol=1e-6), (dpre - grad).abs().max()
+    assert hid.view(-1)[0] == 0 and dpre.view(-1)[0] == 0
+    assert hid.view(-1)[20] == float(pre.view(-1)[20]) and dpre.view(-1)[20] == 1
+
+
 def test_dropout_mask_properties():
     dev = torch.device(DEV)
     m1 = dropout_mask(512, 768, 0.1, seed=1234, offset=0, device=dev)
