@@ -1445,7 +1445,8 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
   const int kt_total = (int)((p.K[0] + BK - 1) / BK);
   int slices = 1;
   if (workspace && tiles < 192) {
-    slices = (int)std::min<int64_t>(std::min<int64_t>(256 / tiles, kt_total / 4), SKINNY_MAX_SLICES);
+    // two workgroups per CU (64 KiB of LDS each): the slices are short and bound by load latency
+    slices = (int)std::min<int64_t>(std::min<int64_t>(512 / tiles, kt_total / 4), SKINNY_MAX_SLICES);
     const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.M * (size_t)p.N * sizeof(float)));
     slices = (int)std::max<int64_t>(1, std::min<int64_t>(slices, fit));
   }
