@@ -5,6 +5,8 @@ block-sparse layout registry and ``ACT2FN``.
 """
 from .blocksparse import (GeneralizedLinear, GeneralizedMatrix, blocksparse_matmul, blocksparse_matmul_backward,
                           get_blocksparse_layout, get_indices_from_layout, register_blocksparse_layout)
+from .checkpoint import (LEGACY_KEY_RENAMES, block_list_to_native, convert_legacy_state_dict, load_reference_state_dict,
+                         native_to_block_list)
 from .ffn import LeanFFN
 from .utils import ACT2FN
 

@@ -9,7 +9,9 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libleanffn.so")
-SOURCES = ["ffn.hip", "elementwise.hip", "gemm_generic.hip", "gemm_mfma_bf16.hip", "profile.hip"]
+# the tiled GEMM kernels are instantiated per epilogue kind in four translation units so that they compile in parallel
+SOURCES = ["gemm_mfma_kind0.hip", "gemm_mfma_kind1.hip", "gemm_mfma_kind2.hip", "gemm_mfma_kind3.hip", "gemm_generic.hip",
+           "elementwise.hip", "ffn.hip", "gemm_mfma_bf16.hip", "profile.hip"]
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_{add,mul,fma}_f32 from scalar float code
 # -pragma-unroll-threshold: the fused GEMM epilogues index the accumulator registers from fully unrolled loops; left rolled
 # (the default threshold is too small for them) the accumulators would be demoted to scratch memory
@@ -43,7 +45,7 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         if verbose and out.strip():
             print(out)
 
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, 8, len(SOURCES))) as pool:
         list(pool.map(compile_one, zip(SOURCES, objects)))
     _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objects, "-o", LIB_PATH])
     return LIB_PATH

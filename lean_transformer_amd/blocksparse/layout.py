@@ -17,26 +17,33 @@ REGISTERED_LAYOUTS = dict()
 
 
 def register_blocksparse_layout(name: str):
-    """Decorator: make ``name(...)`` usable in layout descriptor strings; reference: layout.py:15-21."""
-    def _register(f: callable):
-        if name in REGISTERED_LAYOUTS:
-            logger.warning(f"Overwriting layout {name} with {f}.")
-        REGISTERED_LAYOUTS[name] = f
-        return f
-    return _register
+    """Decorator that files a layout function ``f(out_features, in_features, *args, **kwargs) -> BoolTensor`` under
+    ``name`` so that descriptor strings can call it (same registry as lean_transformer/blocksparse/layout.py:15-21)."""
+    def decorator(layout_fn: callable):
+        previous = REGISTERED_LAYOUTS.get(name)
+        if previous is not None and previous is not layout_fn:
+            logger.warning("layout %r was %s and is now %s", name, previous, layout_fn)
+        REGISTERED_LAYOUTS[name] = layout_fn
+        return layout_fn
+    return decorator
 
 
 def get_blocksparse_layout(out_features: int, in_features: int, layout: str) -> torch.BoolTensor:
-    """Boolean [out_blocks, in_blocks] incidence matrix from a descriptor such as ``pixelfly(block_size=64, stretch=True)``;
-    positional and keyword arguments are forwarded to the registered layout function.  reference: layout.py:24-53."""
-    assert '(' in layout and layout.endswith(')'), "descriptor format must be name(foo=123, bar='456')"
-    parsed = ast.parse(layout).body[0].value
-    name = parsed.func.id
-    args = [ast.literal_eval(arg) for arg in parsed.args]
-    kwargs = {arg.arg: ast.literal_eval(arg.value) for arg in parsed.keywords}
-    if name not in REGISTERED_LAYOUTS:
-        raise ValueError(f"Unknown layout name {name}, supported layouts: {tuple(REGISTERED_LAYOUTS.keys())}")
-    return REGISTERED_LAYOUTS[name](out_features, in_features, *args, **kwargs)
+    """Boolean [out_blocks, in_blocks] incidence matrix from a descriptor such as ``pixelfly(block_size=64, stretch=True)``:
+    a call expression whose literal positional and keyword arguments go to the registered layout function after the two
+    sizes.  reference: layout.py:24-53."""
+    try:
+        call = ast.parse(layout.strip(), mode="eval").body
+    except SyntaxError as e:
+        raise AssertionError(f"layout descriptor {layout!r} is not of the form name(arg, key=value)") from e
+    if not isinstance(call, ast.Call) or not isinstance(call.func, ast.Name):
+        raise AssertionError(f"layout descriptor {layout!r} is not of the form name(arg, key=value)")
+    make = REGISTERED_LAYOUTS.get(call.func.id)
+    if make is None:
+        raise ValueError(f"no layout called {call.func.id!r}; registered: {sorted(REGISTERED_LAYOUTS)}")
+    positional = [ast.literal_eval(node) for node in call.args]
+    named = {kw.arg: ast.literal_eval(kw.value) for kw in call.keywords}
+    return make(out_features, in_features, *positional, **named)
 
 
 def _butterfly_support(size: int, n_factors: int) -> np.ndarray:
@@ -66,18 +73,22 @@ def get_butterfly_layout(out_features: int, in_features: int, block_size: int = 
     cells is stretched over the matrix, a block is active when it overlaps an active cell, and unless ``stretch`` the
     stretched copies along the longer side are regrouped into tiled copies of the square pattern.
     """
+    longer, shorter = max(out_features, in_features), min(out_features, in_features)
+    if longer % shorter:
+        raise AssertionError(f"a {out_features} x {in_features} matrix: the longer side must be a multiple of the shorter")
+    if out_features % block_size or in_features % block_size:
+        raise AssertionError(f"block_size {block_size} does not divide {out_features} x {in_features}")
     if butterfly_size is None:
-        butterfly_size = 2 ** int(math.ceil(math.log2(min(in_features, out_features) / block_size)))
-    assert out_features % in_features == 0 or in_features % out_features == 0, \
-        "if matrix is not square, the longer dimension must be a multiple of the shorter dimension"
-    assert out_features % block_size == 0 and in_features % block_size == 0
-    log_n = int(math.log2(butterfly_size))
-    n_factors = log_n if n_factors is None else n_factors
-    if butterfly_size != 2 ** log_n or butterfly_size < 2:
-        raise NotImplementedError("butterfly_size must be a power of 2")
-    if not (1 <= n_factors <= log_n):
-        raise NotImplementedError("n_factors must be a between 1 and log_2(butterfly_size)")
-    assert out_features % butterfly_size == 0 and in_features % butterfly_size == 0
+        butterfly_size = 1 << max(0, math.ceil(math.log2(shorter / block_size)))
+    log_n = butterfly_size.bit_length() - 1
+    if butterfly_size < 2 or butterfly_size != 1 << log_n:
+        raise NotImplementedError(f"butterfly_size {butterfly_size}: a power of two >= 2 is required")
+    if n_factors is None:
+        n_factors = log_n
+    if not 1 <= n_factors <= log_n:
+        raise NotImplementedError(f"n_factors {n_factors} outside 1 .. log2(butterfly_size) = {log_n}")
+    if out_features % butterfly_size or in_features % butterfly_size:
+        raise AssertionError(f"butterfly_size {butterfly_size} does not divide {out_features} x {in_features}")
     support = _butterfly_support(butterfly_size, n_factors)
     rows_per_cell, cols_per_cell = out_features // butterfly_size, in_features // butterfly_size
     n_out, n_in = out_features // block_size, in_features // block_size
@@ -101,15 +112,16 @@ def get_hypercube_layout(out_features: int, in_features: int, block_size: int, s
     """Pixelfly seen as a hypercube graph, optionally "folded" (an extra edge between antipodal nodes), tiled or stretched
     to a non-square shape.  reference: get_hypercube_layout, layout.py:120-153."""
     smaller = min(out_features, in_features)
-    assert math.log2(smaller / block_size).is_integer(), "layout dimension must be a power of 2"
-    assert out_features % smaller == 0 and in_features % smaller == 0
-    dim = int(math.ceil(math.log2(smaller / block_size)))
+    cells = smaller // block_size
+    if smaller % block_size or cells < 1 or cells & (cells - 1):
+        raise AssertionError(f"hypercube layout: min(out, in) / block_size = {smaller / block_size} must be a power of two")
+    if out_features % smaller or in_features % smaller:
+        raise AssertionError("hypercube layout: the longer side must be a multiple of the shorter")
+    dim = cells.bit_length() - 1
     layout = get_butterfly_layout(smaller, smaller, block_size, n_factors=dim, stretch=False).numpy().copy()
-    assert layout.shape == (2 ** dim, 2 ** dim)
     if folded:
-        nodes = np.arange(2 ** dim)
-        assert not layout[nodes, (2 ** dim - 1) ^ nodes].any()
-        layout[nodes, (2 ** dim - 1) ^ nodes] = True
+        nodes = np.arange(cells)
+        layout[nodes, (cells - 1) ^ nodes] = True  # antipodal node: all dim bits flipped (not an edge of the plain cube)
     ro, ri = out_features // smaller, in_features // smaller
     layout = np.repeat(np.repeat(layout, ro, axis=0), ri, axis=1) if stretch else np.tile(layout, (ro, ri))
     return torch.from_numpy(np.ascontiguousarray(layout))
@@ -125,8 +137,9 @@ def get_indices_from_layout(layout: torch.BoolTensor) -> Tuple[torch.IntTensor, 
     lay = layout.cpu().numpy().astype(bool)
     n_out, n_in = lay.shape
     per_out, per_in = np.unique(lay.sum(1)), np.unique(lay.sum(0))
-    assert len(per_out) == 1, "butterfly layout must have the same number of blocks per row"
-    assert len(per_in) == 1, "butterfly layout must have the same number of blocks per column"
+    if len(per_out) != 1 or len(per_in) != 1:
+        raise AssertionError("unbalanced layout: every block row and every block column must hold the same number of active "
+                             f"blocks (rows hold {per_out.tolist()}, columns {per_in.tolist()})")
     K, A = int(per_out[0]), int(per_in[0])
     out_of_in = np.nonzero(lay.T)[1].reshape(n_in, A)  # ascending output blocks of each input block
     in_of_out = np.nonzero(lay)[1].reshape(n_out, K)  # ascending input blocks of each output block

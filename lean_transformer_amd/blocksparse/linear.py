@@ -15,43 +15,54 @@ from .. import _native as nat
 from .layout import get_blocksparse_layout, get_indices_from_layout
 
 
+def _small_init_std(in_features: int, out_features: int) -> float:
+    """standard deviation the sparse blocks and the shared low-rank factors start from: sqrt(2 / (5 min(fan)))"""
+    return math.sqrt(0.4 / min(in_features, out_features))
+
+
 class GeneralizedMatrix(nn.Module):
-    """A module that stores a shared pytorch tensor for use in GeneralizedLinear layers"""
+    """Weights of one linear map, held apart from the layers that apply it so that several layers can share them.
+
+    ``weight`` is either a dense ``[out_features, in_features]`` matrix (``blocksparse_layout=None``) or the active blocks
+    of a block-sparse one in the "native" order ``[in_features, active blocks per input block, block]`` together with three
+    persistent buffers: the boolean block ``layout`` and the ``forward_indices`` / ``backward_indices`` tables built from
+    it.  ``lowrank_dim > 0`` adds the factors ``lowrank_first [r, in]`` and ``lowrank_second [out, r]`` of an additive
+    low-rank term.  Names and shapes are those of lean_transformer/blocksparse/linear.py:19-66.
+    """
 
     def __init__(self, in_features: int, out_features: int, blocksparse_layout: Optional[str] = None,
                  lowrank_dim: int = 0, blocksparse_backend: str = 'native'):
         super().__init__()
-        self.out_features, self.in_features = out_features, in_features
         if blocksparse_backend != 'native':
             raise NotImplementedError(
                 f"blocksparse_backend={blocksparse_backend!r}: only the 'native' weight format is implemented "
                 "(its matmul runs on HIP kernels; there is no Triton path)")
+        self.in_features, self.out_features = in_features, out_features
         self.blocksparse_backend = blocksparse_backend
+        std = _small_init_std(in_features, out_features)
 
-        if blocksparse_layout is None:
-            # fully-connected weight matrix
-            self.weight = nn.Parameter(torch.empty(out_features, in_features))
-            nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
-            self.layout = self.forward_indices = self.backward_indices = None
-        else:
+        if blocksparse_layout is not None:
             layout = get_blocksparse_layout(out_features, in_features, blocksparse_layout)
-            assert out_features / layout.shape[0] == in_features / layout.shape[1] == in_features // layout.shape[1]
-            block_size = in_features // layout.shape[1]
-            self.register_buffer("layout", layout, persistent=True)
+            out_blocks, in_blocks = layout.shape
+            if in_features % in_blocks or out_features % out_blocks or in_features // in_blocks != out_features // out_blocks:
+                raise AssertionError(f"layout {tuple(layout.shape)} does not cut a {out_features} x {in_features} matrix "
+                                     "into square blocks")
+            block = in_features // in_blocks
             forward_indices, backward_indices = get_indices_from_layout(layout)
-            self.register_buffer("forward_indices", forward_indices, persistent=True)
-            self.register_buffer("backward_indices", backward_indices, persistent=True)
-            active_blocks_per_input = self.forward_indices.numel() // (in_features // block_size)
-            self.weight = nn.Parameter(torch.empty(in_features, active_blocks_per_input, block_size))
-            torch.nn.init.normal_(self.weight, std=math.sqrt(2.0 / (5 * min(out_features, in_features))))
-
-        if lowrank_dim:
-            self.lowrank_first = nn.Parameter(torch.zeros(lowrank_dim, self.in_features))
-            self.lowrank_second = nn.Parameter(torch.zeros(self.out_features, lowrank_dim))
-            nn.init.normal_(self.lowrank_first, std=math.sqrt(2.0 / (5 * min(out_features, in_features))))
-            nn.init.normal_(self.lowrank_second, std=math.sqrt(2.0 / (5 * min(out_features, in_features))))
+            for name, table in (("layout", layout), ("forward_indices", forward_indices),
+                                ("backward_indices", backward_indices)):
+                self.register_buffer(name, table, persistent=True)
+            blocks_per_input = forward_indices.numel() // in_blocks
+            self.weight = nn.Parameter(torch.empty(in_features, blocks_per_input, block).normal_(std=std))
         else:
-            self.lowrank_first = self.lowrank_second = None
+            self.layout = self.forward_indices = self.backward_indices = None
+            self.weight = nn.Parameter(torch.empty(out_features, in_features))
+            nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))  # what nn.Linear does
+
+        self.lowrank_first = self.lowrank_second = None
+        if lowrank_dim:
+            self.lowrank_first = nn.Parameter(torch.empty(lowrank_dim, in_features).normal_(std=std))
+            self.lowrank_second = nn.Parameter(torch.empty(out_features, lowrank_dim).normal_(std=std))
 
     @property
     def shape(self):
@@ -63,59 +74,50 @@ class GeneralizedMatrix(nn.Module):
         return None
 
     def __repr__(self):
-        return f"{self.__class__.__name__}{tuple(self.shape)}"
+        return f"{type(self).__name__}({self.out_features}, {self.in_features})"
 
     def forward(self, input: torch.Tensor, *, ignore_lowrank: bool = False):
-        """
-        Multiply input tensor by this matrix with the same semantics as in torch.nn.Linear(..., bias=False)
-
-        :param ignore_lowrank: if True, the low-rank components (lowrank_dim) will not be used in matrix multiplication
-        """
-        use_lowrank = self.lowrank_first is not None and not ignore_lowrank
-        return _GeneralizedLinear.apply(
-            input, self.weight, None, self.lowrank_first if use_lowrank else None,
-            self.lowrank_second if use_lowrank else None, self.forward_indices, self.backward_indices, None)
+        """``input @ W^T`` like a bias-free ``nn.Linear``; the low-rank term is added unless ``ignore_lowrank``"""
+        first, second = (None, None) if ignore_lowrank else (self.lowrank_first, self.lowrank_second)
+        return _GeneralizedLinear.apply(input, self.weight, None, first, second, self.forward_indices,
+                                        self.backward_indices, None)
 
 
 class GeneralizedLinear(nn.Linear):
-    """A linear layer with a shared full-rank matrix and an individual low-rank adapter"""
+    """``nn.Linear`` look-alike over a (possibly shared) ``GeneralizedMatrix``, with its own bias and an optional low-rank
+    adapter ``adapter_first [a, in]``, ``adapter_second [out, a]`` that belongs to this layer alone
+    (lean_transformer/blocksparse/linear.py:106-149)."""
 
     def __init__(self, matrix: GeneralizedMatrix, adapter_dim: int = 0, bias: bool = True):
-        nn.Module.__init__(self)
+        nn.Module.__init__(self)  # not nn.Linear.__init__: that would allocate a weight of its own
         self.matrix = matrix
-        self.out_features, self.in_features = self.matrix.shape
+        self.out_features, self.in_features = matrix.shape
         self.bias = nn.Parameter(torch.zeros(self.out_features)) if bias else None
-
-        if adapter_dim != 0:
-            self.adapter_first = nn.Parameter(torch.zeros(adapter_dim, self.in_features))
+        self.adapter_first = self.adapter_second = None
+        if adapter_dim:
+            # LoRA-style start (arXiv:2106.09685): random input factor, zero output factor, so the adapter begins as a no-op
+            self.adapter_first = nn.Parameter(nn.init.xavier_normal_(torch.empty(adapter_dim, self.in_features)))
             self.adapter_second = nn.Parameter(torch.zeros(self.out_features, adapter_dim))
-            # initialize in accordance with https://arxiv.org/pdf/2106.09685.pdf
-            nn.init.xavier_normal_(self.adapter_first)
-            nn.init.zeros_(self.adapter_second)
-        else:
-            self.adapter_first = self.adapter_second = None
 
     def get_combined_lowrank_components(self) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-        """Group together low-rank matrices from this layer's adapter and GeneralizedMatrix for faster matmul"""
-        if self.adapter_first is not None and self.matrix.lowrank_first is None:
-            return self.adapter_first, self.adapter_second
-        elif self.adapter_first is None and self.matrix.lowrank_first is not None:
-            return self.matrix.lowrank_first, self.matrix.lowrank_second
-        elif self.adapter_first is not None and self.matrix.lowrank_first is not None:
-            combined_first = torch.cat([self.matrix.lowrank_first, self.adapter_first], dim=0)
-            combined_second = torch.cat([self.matrix.lowrank_second, self.adapter_second], dim=1)
-            return combined_first, combined_second
-        else:
+        """One (first [r + a, in], second [out, r + a]) pair covering the matrix's shared low-rank term and this layer's
+        adapter, so that both ride in a single pair of skinny GEMMs; (None, None) when the layer has neither."""
+        firsts = [t for t in (self.matrix.lowrank_first, self.adapter_first) if t is not None]
+        seconds = [t for t in (self.matrix.lowrank_second, self.adapter_second) if t is not None]
+        if not firsts:
             return None, None
+        if len(firsts) == 1:
+            return firsts[0], seconds[0]
+        return torch.cat(firsts, dim=0), torch.cat(seconds, dim=1)
 
     @property
     def weight(self):
         return self.matrix.weight
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return _GeneralizedLinear.apply(
-            input, self.weight, self.bias, *self.get_combined_lowrank_components(),
-            self.matrix.forward_indices, self.matrix.backward_indices, self.matrix.matmul_op)
+        first, second = self.get_combined_lowrank_components()
+        return _GeneralizedLinear.apply(input, self.weight, self.bias, first, second, self.matrix.forward_indices,
+                                        self.matrix.backward_indices, self.matrix.matmul_op)
 
 
 def compute_dtype_for(weight: torch.Tensor) -> torch.dtype:

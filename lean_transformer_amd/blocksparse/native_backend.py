@@ -18,9 +18,8 @@ def _sparse_desc(weight: torch.Tensor, forward_indices: Optional[torch.Tensor], 
     desc.in_features, desc.out_features = in_features, out_features
     desc.block, desc.blocks_per_in = block, blocks_per_in
     desc.blocks_per_out = (in_features // block) * blocks_per_in // (out_features // block)
-    # the kernels read whichever table their direction needs; the other one may be absent when this is called directly
-    desc.forward_indices = nat.ptr(forward_indices) if forward_indices is not None else nat.ptr(backward_indices)
-    desc.backward_indices = nat.ptr(backward_indices) if backward_indices is not None else nat.ptr(forward_indices)
+    # each direction reads one table (forward: forward_indices, gradients: backward_indices); the other stays NULL
+    desc.forward_indices, desc.backward_indices = nat.ptr(forward_indices), nat.ptr(backward_indices)
     return desc
 
 

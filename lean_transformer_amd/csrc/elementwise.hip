@@ -617,12 +617,7 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   LT_REQUIRE(T > 0 && H > 0 && x && stats && w && dy, LT_ERR_BAD_ARG, "layernorm backward: bad arguments");
   LT_REQUIRE(H <= 256 * LNB_MAXC, LT_ERR_UNSUPPORTED, "layernorm backward: hidden size %d above %d", H, 256 * LNB_MAXC);
   LT_REQUIRE((dweight == nullptr) == (dbias == nullptr), LT_ERR_BAD_ARG, "layernorm backward: pass both dweight and dbias or neither");
-  float* partial = nullptr;
-  if (dweight) {
-    LT_REQUIRE(workspace && workspace_bytes >= lt_ln_backward_workspace(T, H), LT_ERR_WORKSPACE,
-               "layernorm backward: workspace of %zu bytes needed", lt_ln_backward_workspace(T, H));
-    partial = (float*)workspace;
-  }
+  float* partial = dweight ? (float*)workspace : nullptr;
   LtProfileScope scope("layernorm_bwd", 0.0,
                        (double)T * H * ((dx ? 1 : 0) + (dweight ? 1 : 0)) * (lt_dtype_size(x_dtype) + lt_dtype_size(dy_dtype)) +
                            (double)T * H * ((dx ? lt_dtype_size(dx_dtype) : 0) + (dx && residual_grad ? lt_dtype_size(dx_dtype) : 0)),
@@ -631,7 +626,13 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   const bool vec = (H & 3) == 0 && H <= 64 * 4 * LN_MAXV && lt_aligned(x, 16) && lt_aligned(dy, 16) && lt_aligned(w, 16) &&
                    (!dx || lt_aligned(dx, 16)) && (!residual_grad || lt_aligned(residual_grad, 16)) &&
                    (!partial || lt_aligned(partial, 16));
-  int partial_rows;
+  // partial (dweight, dbias) rows of the path taken: one pair per row slice (vectorised) or per workgroup (any-shape)
+  int partial_rows = vec ? ln_bwd_slices(T) : ln_bwd_blocks(T);
+  if (dweight) {
+    const size_t need = (size_t)partial_rows * 2 * (size_t)H * sizeof(float);
+    LT_REQUIRE(workspace && workspace_bytes >= need, LT_ERR_WORKSPACE,
+               "layernorm backward: %zu bytes of scratch needed for the parameter gradients, %zu given", need, workspace_bytes);
+  }
   if (vec) {
     if (dx) {
       dim3 grid(blocks_for(T, 4)), block(256);
@@ -659,7 +660,6 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
 #undef LT_LNB_DX_V
       LT_LAUNCH_CHECK();
     }
-    partial_rows = ln_bwd_slices(T);
     if (partial) {
       const int64_t rps = (T + partial_rows - 1) / partial_rows;
       dim3 grid(blocks_for(H, 256), partial_rows), block(256);
@@ -676,7 +676,6 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
       LT_LAUNCH_CHECK();
     }
   } else {
-    partial_rows = ln_bwd_blocks(T);
     dim3 grid(partial_rows), block(256);
 #define LT_LNB_LAUNCH(TX, TDY, TDX)                                                                                      \
   hipLaunchKernelGGL((ln_bwd_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \

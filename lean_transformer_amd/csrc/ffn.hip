@@ -47,13 +47,17 @@ int check_dtype(int d, const char* what) {
   return LT_OK;
 }
 
-int check_linear(const lt_linear& lin, const char* name) {
+// which index tables a call reads: the forward walk takes forward_indices, both gradient walks take backward_indices
+enum { NEED_FWD_TABLE = 1, NEED_BWD_TABLE = 2 };
+
+int check_linear(const lt_linear& lin, const char* name, int tables = NEED_FWD_TABLE | NEED_BWD_TABLE) {
   LT_REQUIRE(lin.weight && lin.in_features > 0 && lin.out_features > 0, LT_ERR_BAD_ARG, "%s: weight / sizes missing", name);
   LT_REQUIRE(lin.lowrank >= 0 && ((lin.lowrank > 0) == (lin.lowrank_first != nullptr)) &&
                  ((lin.lowrank > 0) == (lin.lowrank_second != nullptr)),
              LT_ERR_BAD_ARG, "%s: lowrank=%d does not match the low-rank pointers", name, lin.lowrank);
   if (lin.block > 0) {
-    LT_REQUIRE(lin.forward_indices && lin.backward_indices, LT_ERR_BAD_ARG, "%s: sparse weight without index tables", name);
+    LT_REQUIRE(!(tables & NEED_FWD_TABLE) || lin.forward_indices, LT_ERR_BAD_ARG, "%s: sparse weight without forward_indices", name);
+    LT_REQUIRE(!(tables & NEED_BWD_TABLE) || lin.backward_indices, LT_ERR_BAD_ARG, "%s: sparse weight without backward_indices", name);
     LT_REQUIRE(lin.in_features % lin.block == 0 && lin.out_features % lin.block == 0, LT_ERR_BAD_ARG,
                "%s: features not divisible by block %d", name, lin.block);
     LT_REQUIRE(lin.blocks_per_in > 0 && lin.blocks_per_out > 0 &&
@@ -237,6 +241,8 @@ int check_ffn_desc(const lt_ffn_desc* d) {
              (long long)d->tokens, d->hidden, d->intermediate);
   LT_TRY(check_dtype(d->io_dtype, "ffn io_dtype"));
   LT_TRY(check_dtype(d->compute_dtype, "ffn compute_dtype"));
+  // the LayerNorm kernels hold a row in registers (backward has no strided variant): refuse wider rows before any work
+  LT_REQUIRE(d->hidden <= 8192, LT_ERR_UNSUPPORTED, "ffn: hidden size %d exceeds 8192, the widest row the LayerNorm kernels take", d->hidden);
   LT_REQUIRE(d->act >= LT_ACT_GELU_FUSED && d->act <= LT_ACT_SILU, LT_ERR_UNSUPPORTED, "ffn: unknown activation %d", d->act);
   LT_REQUIRE(d->ln_weight && d->ln_bias, LT_ERR_BAD_ARG, "ffn: LayerNorm parameters missing");
   LT_REQUIRE((d->post_ln_weight == nullptr) == (d->post_ln_bias == nullptr), LT_ERR_BAD_ARG, "ffn: post-LN needs weight and bias");
@@ -461,7 +467,7 @@ extern "C" int lt_linear_forward(const lt_linear* lin, int64_t tokens, int32_t d
                                  void* lowrank_hid, void* stream) {
   LT_REQUIRE(lin && x && y && tokens > 0, LT_ERR_BAD_ARG, "linear forward: bad arguments");
   LT_TRY(check_dtype(dtype, "linear forward"));
-  LT_TRY(check_linear(*lin, "linear"));
+  LT_TRY(check_linear(*lin, "linear", NEED_FWD_TABLE));
   EpiParams e = epi_store_params(y, lin->out_features, dtype, lin->bias);
   return linear_forward_impl(*lin, tokens, dtype, x, EPI_STORE, e, lowrank_hid, dtype, (hipStream_t)stream);
 }
@@ -471,7 +477,7 @@ extern "C" int lt_linear_backward(const lt_linear* lin, int64_t tokens, int32_t 
                                   size_t workspace_bytes, void* stream) {
   LT_REQUIRE(lin && x && dy && grads && tokens > 0, LT_ERR_BAD_ARG, "linear backward: bad arguments");
   LT_TRY(check_dtype(dtype, "linear backward"));
-  LT_TRY(check_linear(*lin, "linear"));
+  LT_TRY(check_linear(*lin, "linear", NEED_BWD_TABLE));
   LT_REQUIRE(workspace && lt_aligned(workspace, 256) &&
                  workspace_bytes >= lt_linear_backward_workspace_bytes(lin, tokens, dtype),
              LT_ERR_WORKSPACE, "linear backward: needs a 256-byte aligned workspace of %zu bytes",
@@ -499,7 +505,7 @@ extern "C" int lt_blocksparse_forward(const lt_linear* lin, int64_t tokens, int3
   LT_REQUIRE(lin->block > 0, LT_ERR_BAD_ARG, "blocksparse forward: dense weight");
   LT_TRY(check_dtype(dtype, "blocksparse forward"));
   const lt_linear l = main_weight_only(*lin);
-  LT_TRY(check_linear(l, "blocksparse"));
+  LT_TRY(check_linear(l, "blocksparse", NEED_FWD_TABLE));
   EpiParams e = epi_store_params(y, l.out_features, dtype, nullptr);
   return linear_forward_impl(l, tokens, dtype, x, EPI_STORE, e, nullptr, dtype, (hipStream_t)stream);
 }
@@ -510,7 +516,7 @@ extern "C" int lt_blocksparse_backward(const lt_linear* lin, int64_t tokens, int
   LT_REQUIRE(lin->block > 0, LT_ERR_BAD_ARG, "blocksparse backward: dense weight");
   LT_TRY(check_dtype(dtype, "blocksparse backward"));
   const lt_linear l = main_weight_only(*lin);
-  LT_TRY(check_linear(l, "blocksparse"));
+  LT_TRY(check_linear(l, "blocksparse", NEED_BWD_TABLE));
   lt_linear_grads grads;
   memset(&grads, 0, sizeof(grads));
   grads.weight = dweight;
@@ -582,8 +588,6 @@ extern "C" int lt_gemm(int32_t dtype, int64_t m, int64_t n, int64_t k, const voi
   p.krot = force_generic >> 4;
   force_generic &= 15;
   if (force_generic == 1) return lt_launch_gemm_generic(p, EPI_STORE, dtype, dtype, (hipStream_t)stream);
-  lt_gemm_set_mfma_variant(force_generic == 2 ? 1 : 0);  // 2: the register-staged tiled kernel instead of the copy-based one
-  const int status = lt_launch_gemm(p, EPI_STORE, dtype, dtype, (hipStream_t)stream);
-  lt_gemm_set_mfma_variant(0);
-  return status;
+  p.variant = force_generic == 2 ? 1 : 0;  // 2: the register-staged tiled kernel instead of the copy-based one
+  return lt_launch_gemm(p, EPI_STORE, dtype, dtype, (hipStream_t)stream);
 }

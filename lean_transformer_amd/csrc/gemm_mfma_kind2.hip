@@ -1,0 +1,10 @@
+// Instantiates the tiled bf16 GEMM kernels with the EPI_ACT_BWD epilogue (dense layouts and block-sparse walks).
+#include "gemm_mfma_kernels.h"
+
+int lt_mfma_launch_dense_kind2(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+  return launch_layout<EPI_ACT_BWD>(p, io_dtype, stream);
+}
+
+int lt_mfma_launch_sparse_kind2(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+  return launch_sparse<EPI_ACT_BWD>(p, io_dtype, stream);
+}

@@ -78,6 +78,7 @@ struct GemmProblem {
   int ksplit;
   int64_t split_stride;
   int krot;  // copy-based kernel: how workgroups stagger their walk over k (0: all start at k = 0)
+  int variant;  // tiled bf16 kernels: 0 the launcher's choice, 1 the register-staged kernel where the copy-based one applies
 };
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -481,7 +482,5 @@ int lt_launch_gemm_out(const GemmProblem& p, int dtype, int io_dtype, void* work
 // out[i] = sum_s partial[s * stride + i] (+ bias[i % cols]) for i < count, cast to out_dtype
 int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t count, int cols, const float* bias,
                      int out_dtype, void* out, hipStream_t stream);
-// 0: choose; 1: register-staged tiled kernel; 2: copy-based tiled kernel
-void lt_gemm_set_mfma_variant(int v);
 // picks the tiled kernel when it applies and dtype is bf16, else the any-shape kernel
 int lt_launch_gemm(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);

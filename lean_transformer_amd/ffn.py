@@ -19,21 +19,25 @@ from .utils import ACT2FN, ACT_KINDS, activation_kind
 
 
 class LeanFFN(nn.Module):
-    """
-    A transformer FFN module that doesn't hog your GPU memory. Uses a manually optimized differentiation algorithm.
+    """Pre-LayerNorm feed-forward block  y = [x +] dropout([postLN](act(LN(x) W1^T + b1) W2^T + b2))  whose backward keeps
+    only x and the pre-activation alive and rebuilds everything else inside the HIP kernels.
 
-    :param hidden_size: base hidden size of the transformer
-    :param intermediate_size: a (typically larger) hidden dimension where activation is applied
-    :param activation: a pytorch nonlinearity to use in the intermediate layer
-    :param gated: use gated activations based on https://arxiv.org/abs/2002.05202 and https://arxiv.org/abs/2102.11972
-      note: gated activations require 1.5x more parameters compared to their non-gated variants.
-    :param layer_norm_eps: see torch.nn.functional.layer_norm
-    :param post_layer_norm: if set, applies an additional layer norm to projected attention outputs before residuals
-    :param dropout: hidden dropout probability, applied to the output projection (before adding residual)
-    :param residual: if True, adds the original layer input to the final layer output
-    :param ffn_custom_grad: if True (default), use the fused HIP forward/backward that saves memory
-    :param i2h_proj: custom *first* linear layer (hidden_size -> intermediate_size or 2x indermediate_size)
-    :param h2o_proj: custom *second* linear layer (intermediate_size -> hidden_size)
+    The constructor, the attribute names and the parameter names follow lean_transformer/ffn.py:35-64 so that models and
+    checkpoints written for that class work with this one.
+
+    hidden_size        width of the residual stream (input and output)
+    intermediate_size  width of the activation; the first projection is twice as wide when ``gated``
+    activation         element-wise nonlinearity; on the kernel path it must be one that ``utils.activation_kind`` knows
+    gated              GLU variant: the first half of the up-projection passes through ``activation`` and multiplies the
+                       second half (arXiv:2002.05202); costs 1.5x the parameters of the plain block
+    layer_norm_eps     epsilon of both LayerNorms
+    dropout            drop probability on the block's output, before the residual is added; training mode only
+    post_layer_norm    second LayerNorm right after the down-projection (CogView / NormFormer style)
+    i2h_proj, h2o_proj projections to use instead of fresh ``nn.Linear`` layers (hidden -> intermediate[*2] and
+                       intermediate -> hidden); the kernel path takes ``nn.Linear`` and ``GeneralizedLinear`` exactly
+    residual           add the input to the output
+    ffn_custom_grad    True: one fused library call forward and one backward (memory-lean).  False: the same maths as a
+                       chain of stock PyTorch ops differentiated by autograd.  May be flipped at any time.
     """
 
     def __init__(
@@ -51,71 +55,69 @@ class LeanFFN(nn.Module):
         ffn_custom_grad: bool = True,
     ):
         super().__init__()
-        i2h_out_features = intermediate_size * 2 if gated else intermediate_size
-        self.i2h_proj = nn.Linear(hidden_size, i2h_out_features) if i2h_proj is None else i2h_proj
-        self.h2o_proj = nn.Linear(intermediate_size, hidden_size) if h2o_proj is None else h2o_proj
-        if ffn_custom_grad:
-            assert type(self.i2h_proj) in (nn.Linear, GeneralizedLinear), "custom grad supports only nn.Linear and GeneralizedLinear"
-            assert type(self.h2o_proj) in (nn.Linear, GeneralizedLinear), "custom grad supports only nn.Linear and GeneralizedLinear"
-        assert self.i2h_proj.in_features == self.h2o_proj.out_features == hidden_size
-        assert self.i2h_proj.out_features == i2h_out_features and self.h2o_proj.in_features == intermediate_size
+        up_width = 2 * intermediate_size if gated else intermediate_size
+        self.i2h_proj = i2h_proj if i2h_proj is not None else nn.Linear(hidden_size, up_width)
+        self.h2o_proj = h2o_proj if h2o_proj is not None else nn.Linear(intermediate_size, hidden_size)
+        for name, proj, fan_in, fan_out in (("i2h_proj", self.i2h_proj, hidden_size, up_width),
+                                            ("h2o_proj", self.h2o_proj, intermediate_size, hidden_size)):
+            if ffn_custom_grad and type(proj) not in (nn.Linear, GeneralizedLinear):
+                raise AssertionError(f"{name} is a {type(proj).__name__}: the fused path runs nn.Linear and GeneralizedLinear "
+                                     "projections only (pass ffn_custom_grad=False for other layer types)")
+            if (proj.in_features, proj.out_features) != (fan_in, fan_out):
+                raise AssertionError(f"{name} maps {proj.in_features} -> {proj.out_features} features, "
+                                     f"this block needs {fan_in} -> {fan_out}")
         self.pre_layer_norm = nn.LayerNorm(hidden_size, eps=layer_norm_eps)
         self.post_layer_norm = nn.LayerNorm(hidden_size, eps=layer_norm_eps) if post_layer_norm else None
-        self.activation = activation
-        self.gated = gated
-        self.dropout = dropout
-        self.residual = residual
+        self.activation, self.gated = activation, gated
+        self.dropout, self.residual = dropout, residual
         self.ffn_custom_grad = ffn_custom_grad
 
     def forward(self, input):
-        return self._forward_custom(input) if self.ffn_custom_grad else self._forward_pytorch(input)
+        if self.ffn_custom_grad:
+            return self._forward_custom(input)
+        return self._forward_pytorch(input)
 
     def _forward_pytorch(self, input):
-        input_2d = input.view(-1, input.shape[-1])
-        input_ln = F.layer_norm(
-            input_2d, input.shape[-1:], self.pre_layer_norm.weight, self.pre_layer_norm.bias, self.pre_layer_norm.eps
-        )
-        pre_activation = self.i2h_proj(input_ln)
-        hid_act = _LeanFFN._apply_activation(pre_activation, self.activation, gated=self.gated)
-
-        out = self.h2o_proj(hid_act)
-        if self.post_layer_norm:
+        """The block as stock PyTorch ops under autograd (lean_transformer/ffn.py:69-85).  On a GPU the dropout mask is
+        the Philox stream the fused path would draw from the same generator state, so both settings of ``ffn_custom_grad``
+        drop the same elements under one seed."""
+        width = input.shape[-1]
+        rows = input.view(-1, width)
+        ln = self.pre_layer_norm
+        normed = F.layer_norm(rows, (width,), ln.weight, ln.bias, ln.eps)
+        hidden_act = _LeanFFN._apply_activation(self.i2h_proj(normed), self.activation, gated=self.gated)
+        out = self.h2o_proj(hidden_act)
+        if self.post_layer_norm is not None:
             out = self.post_layer_norm(out)
-
-        if self.dropout and self.training:
-            out = torch.dropout(out, self.dropout, self.training)
+        if self.training and self.dropout:
+            if out.is_cuda:
+                keep = philox_keep_mask(out.shape[0], width, float(self.dropout), out.device)
+                out = out * (keep.to(out.dtype) * (1.0 / (1.0 - float(self.dropout))))
+            else:
+                out = torch.dropout(out, self.dropout, True)
         if self.residual:
-            out = out + input_2d
+            out = out + rows
         return out.view(*input.shape)
 
-    def _forward_custom(self, input):
-        post_ln_weight = post_ln_bias = None
-        if self.post_layer_norm is not None:
-            post_ln_weight, post_ln_bias = self.post_layer_norm.weight, self.post_layer_norm.bias
-        i2h_lowrank_first = i2h_lowrank_second = h2o_lowrank_first = h2o_lowrank_second = None
-        i2h_forward_indices = i2h_backward_indices = h2o_forward_indices = h2o_backward_indices = None
-        i2h_matmul_op = h2o_matmul_op = None
-        if isinstance(self.i2h_proj, GeneralizedLinear):
-            i2h_lowrank_first, i2h_lowrank_second = self.i2h_proj.get_combined_lowrank_components()
-            i2h_forward_indices = self.i2h_proj.matrix.forward_indices
-            i2h_backward_indices = self.i2h_proj.matrix.backward_indices
-            i2h_matmul_op = self.i2h_proj.matrix.matmul_op
-        if isinstance(self.h2o_proj, GeneralizedLinear):
-            h2o_lowrank_first, h2o_lowrank_second = self.h2o_proj.get_combined_lowrank_components()
-            h2o_forward_indices = self.h2o_proj.matrix.forward_indices
-            h2o_backward_indices = self.h2o_proj.matrix.backward_indices
-            h2o_matmul_op = self.h2o_proj.matrix.matmul_op
+    @staticmethod
+    def _projection_extras(proj):
+        """(lowrank_first, lowrank_second, forward_indices, backward_indices, matmul_op) of a projection; a plain
+        ``nn.Linear`` has none of them"""
+        if not isinstance(proj, GeneralizedLinear):
+            return None, None, None, None, None
+        first, second = proj.get_combined_lowrank_components()
+        return first, second, proj.matrix.forward_indices, proj.matrix.backward_indices, proj.matrix.matmul_op
 
+    def _forward_custom(self, input):
+        """Flattens the module state into the 25 positional arguments of ``_LeanFFN.apply`` (order of
+        lean_transformer/ffn.py:105-131)."""
+        post = self.post_layer_norm
         return _LeanFFN.apply(
-            input,
-            self.pre_layer_norm.weight, self.pre_layer_norm.bias,
-            self.i2h_proj.weight, self.i2h_proj.bias, i2h_lowrank_first, i2h_lowrank_second,
-            i2h_forward_indices, i2h_backward_indices, i2h_matmul_op,
-            self.h2o_proj.weight, self.h2o_proj.bias, h2o_lowrank_first, h2o_lowrank_second,
-            h2o_forward_indices, h2o_backward_indices, h2o_matmul_op,
-            post_ln_weight, post_ln_bias,
-            self.activation, self.gated, self.dropout, self.training, self.pre_layer_norm.eps, self.residual,
-        )
+            input, self.pre_layer_norm.weight, self.pre_layer_norm.bias,
+            self.i2h_proj.weight, self.i2h_proj.bias, *self._projection_extras(self.i2h_proj),
+            self.h2o_proj.weight, self.h2o_proj.bias, *self._projection_extras(self.h2o_proj),
+            None if post is None else post.weight, None if post is None else post.bias,
+            self.activation, self.gated, self.dropout, self.training, self.pre_layer_norm.eps, self.residual)
 
 
 def _draw_dropout_stream(device: torch.device, numel: int):
@@ -127,16 +129,27 @@ def _draw_dropout_stream(device: torch.device, numel: int):
     return seed, offset
 
 
+def philox_keep_mask(tokens: int, hidden: int, p: float, device: torch.device) -> torch.Tensor:
+    """uint8 keep-mask [tokens, hidden] of the next dropout sub-stream of ``device``'s generator (which it advances): the
+    elements the fused forward epilogue would keep had it drawn that sub-stream"""
+    seed, offset = _draw_dropout_stream(device, tokens * hidden)
+    keep = torch.empty(tokens, hidden, dtype=torch.uint8, device=device)
+    if tokens > 0:
+        nat.check(nat.lib().lt_dropout_mask(tokens, hidden, p, seed, offset, nat.ptr(keep), nat.current_stream(device)),
+                  "lt_dropout_mask")
+    return keep
+
+
 class _LeanFFN(torch.autograd.Function):
     """Autograd function for transformer FFN: one library call forward, one backward."""
 
     @staticmethod
     def _apply_activation(pre_activation: torch.Tensor, activation: callable, gated: bool):
-        if not gated:
-            return activation(pre_activation)
-        else:
-            pre_gate, lin = pre_activation.split(pre_activation.shape[-1] // 2, dim=-1)
-            return activation(pre_gate).mul_(lin)
+        """stock-op activation of the up-projection's output; gated: act(first half) * second half (ffn.py:138-144)"""
+        if gated:
+            gate, linear = pre_activation.chunk(2, dim=-1)
+            return activation(gate) * linear
+        return activation(pre_activation)
 
     @staticmethod
     def forward(

@@ -111,6 +111,12 @@ class FFNConfig:
     ln_eps: float = 1e-12
     residual: bool = True
     dropout: float = 0.0  # probability; the mask is passed separately
+    # Round the LayerNorm output, the pre-activation and the activation output to bfloat16 (straight-through for autograd):
+    # the three places where the reference stores a bf16 tensor under torch.autocast(bfloat16) -- layer_norm runs in fp32 and
+    # its result is cast at the linear's input, the linear's output P is bf16, the activation's output is bf16 (ffn.py:184-191
+    # under autocast).  Off: everything in the dtype of the inputs.  Needed to compare a bf16 run where the activation's
+    # derivative jumps (relu): there the derivative depends on the sign of the *stored* P, not of its exact value.
+    bf16_rounding: bool = False
 
 
 @dataclass
@@ -130,6 +136,11 @@ class FFNParams:
         return out
 
 
+def round_bf16_straight_through(t: torch.Tensor) -> torch.Tensor:
+    """value of t rounded to bfloat16 (round-to-nearest-even, as a cast does), gradient of the identity"""
+    return t + (t.to(torch.bfloat16).to(t.dtype) - t).detach()
+
+
 def apply_activation(pre_activation: torch.Tensor, act: str, gated: bool) -> torch.Tensor:
     """reference: _LeanFFN._apply_activation, ffn.py:138-144 -- the FIRST half of the features is the gate."""
     if not gated:
@@ -146,9 +157,10 @@ def plain_ffn(x: torch.Tensor, p: FFNParams, keep_mask: Optional[torch.Tensor] =
     """
     cfg = p.cfg
     x2d = x.reshape(-1, x.shape[-1])
-    u = F.layer_norm(x2d, x2d.shape[-1:], p.ln_weight, p.ln_bias, cfg.ln_eps)
-    pre = linear_forward(u, p.i2h)
-    h = apply_activation(pre, cfg.act, cfg.gated)
+    rnd = round_bf16_straight_through if cfg.bf16_rounding else (lambda t: t)
+    u = rnd(F.layer_norm(x2d, x2d.shape[-1:], p.ln_weight, p.ln_bias, cfg.ln_eps))
+    pre = rnd(linear_forward(u, p.i2h))
+    h = rnd(apply_activation(pre, cfg.act, cfg.gated))
     out = linear_forward(h, p.h2o)
     if p.post_ln_weight is not None:
         out = F.layer_norm(out, out.shape[-1:], p.post_ln_weight, p.post_ln_bias, cfg.ln_eps)

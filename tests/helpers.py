@@ -22,7 +22,7 @@ def oracle_linear(proj, device, dtype) -> offn.LinearParams:
     return offn.LinearParams(leaf(proj.weight), leaf(proj.bias), out_features=proj.out_features)
 
 
-def oracle_params(ffn: "lt.LeanFFN", device="cpu", dtype=torch.float32) -> offn.FFNParams:
+def oracle_params(ffn: "lt.LeanFFN", device="cpu", dtype=torch.float32, bf16_rounding=False) -> offn.FFNParams:
     """fp32 (or fp64) leaf copies of a module's parameters, in the oracle's container"""
     def leaf(t):
         return None if t is None else t.detach().to(device=device, dtype=dtype).clone().requires_grad_(True)
@@ -33,7 +33,8 @@ def oracle_params(ffn: "lt.LeanFFN", device="cpu", dtype=torch.float32) -> offn.
         oracle_linear(ffn.i2h_proj, device, dtype), oracle_linear(ffn.h2o_proj, device, dtype),
         leaf(post.weight) if post is not None else None, leaf(post.bias) if post is not None else None,
         offn.FFNConfig(gated=ffn.gated, act=activation_kind(ffn.activation), ln_eps=ffn.pre_layer_norm.eps,
-                       residual=ffn.residual, dropout=ffn.dropout if ffn.training else 0.0))
+                       residual=ffn.residual, dropout=ffn.dropout if ffn.training else 0.0,
+                       bf16_rounding=bf16_rounding))
 
 
 def module_tensors(ffn: "lt.LeanFFN"):

@@ -26,8 +26,8 @@ def _run_module(ffn, x, dy):
     return y.detach(), grads[0], list(grads[1:])
 
 
-def _compare(ffn, x_cpu, dy_cpu, dtype, oracle_device="cpu", mask=None):
-    p = oracle_params(ffn, oracle_device)
+def _compare(ffn, x_cpu, dy_cpu, dtype, oracle_device="cpu", mask=None, bf16_rounding=False):
+    p = oracle_params(ffn, oracle_device, bf16_rounding=bf16_rounding)
     y_ref, dx_ref, g_ref = run_oracle(p, x_cpu.float().to(oracle_device), dy_cpu.float().to(oracle_device), mask)
     y, dx, g = _run_module(ffn, x_cpu.to(DEV), dy_cpu.to(DEV))
     assert_close(y, y_ref, dtype, "y")
@@ -377,7 +377,7 @@ def _full_size_checks(ffn, x, dy, mask_p):
     mask = dropout_mask(tokens, hidden, mask_p, seed, offset, torch.device(DEV)) if mask_p > 0 else None
     # (1) the oracle, evaluated in fp32 on the GPU, on the bf16-rounded weights
     p = oracle_params(ffn, DEV)
-    y_ref, dx_ref, g_ref = run_oracle(p, x.to(DEV), dy.to(DEV), mask)
+    y_ref, dx_ref, g_ref = run_oracle(p, x.float().to(DEV), dy.float().to(DEV), mask)
     assert_close(y, y_ref, torch.bfloat16, "y")
     assert_close(dx, dx_ref, torch.bfloat16, "dx")
     for i, (a, b) in enumerate(zip(g, g_ref)):
@@ -386,7 +386,7 @@ def _full_size_checks(ffn, x, dy, mask_p):
     # (2) rows are independent: 128 rows through the oracle on the CPU
     rows = torch.randperm(tokens, generator=torch.Generator().manual_seed(1))[:128]
     p_cpu = oracle_params(ffn, "cpu")
-    x2, dy2 = x.reshape(tokens, hidden)[rows], dy.reshape(tokens, hidden)[rows]
+    x2, dy2 = x.float().reshape(tokens, hidden)[rows], dy.float().reshape(tokens, hidden)[rows]
     y_cpu, dx_cpu, _ = run_oracle(p_cpu, x2, dy2, None if mask is None else mask.cpu()[rows])
     assert_close(y.reshape(tokens, hidden)[rows.to(DEV)], y_cpu, torch.bfloat16, "y rows")
     assert_close(dx.reshape(tokens, hidden)[rows.to(DEV)], dx_cpu, torch.bfloat16, "dx rows")

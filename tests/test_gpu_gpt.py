@@ -40,43 +40,84 @@ def test_small_model_fp32():
         assert_close(grads[name], grads_ref[name], torch.float32, name)
 
 
+def _print_table(label, table):
+    print(f"{label}: per gradient, max relative error / cosine against the fp32 run; last pair: hip bf16 against stock bf16")
+    for name, e_hip, c_hip, e_stock, c_stock, e_pair, c_pair in table:
+        print(f"  {name:58s} hip {e_hip:.3e} {c_hip:.6f} | stock bf16 {e_stock:.3e} {c_stock:.6f} | pair {e_pair:.3e} {c_pair:.6f}")
+    worst = max(table, key=lambda r: r[1])
+    print(f"{label} worst hip-vs-fp32 gradient: {worst[0]} {worst[1]:.3e} / {worst[2]:.6f}; stock bf16 there {worst[3]:.3e} / {worst[4]:.6f}")
+
+
+def _bf16_against_fp32_truth(hip, ref, ids, label, loss_tol=1e-3):
+    """Three runs of the same weights on the same batch: the FFN on the HIP kernels under bf16 autocast, the stock-op model
+    under bf16 autocast, and the stock-op model in fp32 without autocast as ground truth.  Two bf16 runs of a deep model
+    differ from each other by rounding noise, so each is measured against the fp32 run and the HIP run must be no further
+    from the truth than the stock-op bf16 run is:
+      * averaged over the gradient tensors, max relative error and 1 - cosine of the HIP run <= 1.05 x the stock run's;
+      * per tensor <= 1.6 x (max relative error) and <= 1.4 x (1 - cosine): the per-tensor figures are maxima over a few
+        hundred to a few million elements and scatter by about +-50 % between any two bf16 runs.
+    Returns the per-tensor table [(name, err_hip, cos_hip, err_stock, cos_stock, err_hip_vs_stock, cos_hip_vs_stock)]."""
+    loss_hip, g_hip = _train_step(hip, ids, autocast=True)
+    loss_bf16, g_bf16 = _train_step(ref, ids, autocast=True)
+    loss_fp32, g_fp32 = _train_step(ref, ids, autocast=False)
+    print(f"{label} loss: hip bf16 {loss_hip.item():.6f}  stock bf16 {loss_bf16.item():.6f}  stock fp32 {loss_fp32.item():.6f}")
+    assert abs(loss_hip.item() - loss_bf16.item()) <= loss_tol * abs(loss_bf16.item())
+    assert abs(loss_hip.item() - loss_fp32.item()) <= 1.25 * abs(loss_bf16.item() - loss_fp32.item()) + 1e-4 * abs(loss_fp32.item())
+    assert g_hip.keys() == g_bf16.keys() == g_fp32.keys()
+    table = []
+    for name in g_hip:
+        assert torch.isfinite(g_hip[name]).all(), name
+        truth = g_fp32[name]
+        row = (name, rel_err(g_hip[name], truth), cosine(g_hip[name], truth), rel_err(g_bf16[name], truth),
+               cosine(g_bf16[name], truth), rel_err(g_hip[name], g_bf16[name]), cosine(g_hip[name], g_bf16[name]))
+        table.append(row)
+    _print_table(label, table)
+    n = len(table)
+    mean_err_hip, mean_err_stock = sum(r[1] for r in table) / n, sum(r[3] for r in table) / n
+    mean_ang_hip, mean_ang_stock = sum(1 - r[2] for r in table) / n, sum(1 - r[4] for r in table) / n
+    print(f"{label} mean over {n} gradients: max relative error hip {mean_err_hip:.3e} stock bf16 {mean_err_stock:.3e}; "
+          f"1 - cosine hip {mean_ang_hip:.3e} stock bf16 {mean_ang_stock:.3e}")
+    assert mean_err_hip <= 1.05 * mean_err_stock and mean_ang_hip <= 1.05 * mean_ang_stock
+    for name, e_hip, c_hip, e_stock, c_stock, e_pair, c_pair in table:
+        assert e_hip <= 1.6 * e_stock + 1e-4, f"{name}: hip {e_hip:.3e} vs truth, stock bf16 {e_stock:.3e} vs truth"
+        assert 1.0 - c_hip <= 1.4 * (1.0 - c_stock) + 1e-6, f"{name}: cosine hip {c_hip:.6f}, stock bf16 {c_stock:.6f}"
+    return table
+
+
 @pytest.mark.parametrize("autocast", [False, True])
 def test_small_model_attention_projections_on_the_hip_linear_layer(autocast):
     """the attention's qkv and output projections as GeneralizedLinear on the HIP kernels too (the layer type the reference
-    builds there), FFN on the HIP kernels: loss and every gradient against the all-stock model"""
+    builds there), FFN on the HIP kernels: loss and every gradient against the all-stock model; under bf16 autocast both
+    are measured against the stock model's fp32 run"""
     cfg = GPTConfig(vocab_size=1000, embedding_size=192, hidden_size=256, num_layers=2, num_heads=4,
                     intermediate_size=512, layer_norm_eps=1e-5)
     hip, ref = _pair(cfg, linear_impl="hip")
     ids = torch.randint(0, cfg.vocab_size, (2, 128), generator=torch.Generator().manual_seed(1)).to(DEV)
-    loss, grads = _train_step(hip, ids, autocast=autocast)
-    loss_ref, grads_ref = _train_step(ref, ids, autocast=autocast)
-    assert abs(loss.item() - loss_ref.item()) <= (1e-3 if autocast else 1e-5) * abs(loss_ref.item())
+    if autocast:  # two layers deep, the two bf16 runs also meet the bf16 bar against each other, tensor by tensor
+        for name, _, _, _, _, e_pair, c_pair in _bf16_against_fp32_truth(hip, ref, ids, "small model"):
+            assert e_pair <= 2e-2 and c_pair >= 0.9999, f"{name}: hip bf16 against stock bf16 {e_pair:.3e} / {c_pair:.6f}"
+        return
+    loss, grads = _train_step(hip, ids, autocast=False)
+    loss_ref, grads_ref = _train_step(ref, ids, autocast=False)
+    assert abs(loss.item() - loss_ref.item()) <= 1e-5 * abs(loss_ref.item())
     assert grads.keys() == grads_ref.keys()
     for name in grads:
-        if autocast:
-            err, cos = rel_err(grads[name], grads_ref[name]), cosine(grads[name], grads_ref[name])
-            assert err <= 5e-2 and cos >= 0.999, f"{name}: max relative error {err:.3e}, cosine {cos:.6f}"
-        else:
-            assert_close(grads[name], grads_ref[name], torch.float32, name)
+        assert_close(grads[name], grads_ref[name], torch.float32, name)
 
 
 def test_config5_bf16_train_step():
     """vocab 10000, hidden 768, 12 layers, 16 heads, rotary, GeGLU 3072, tied embeddings, ids [16, 1024], labels = ids,
-    bf16 autocast over fp32 parameters and an fp32 residual stream.  Twelve layers of bf16 rounding separate the two runs,
-    so the per-tensor bar is the bf16 one (max relative error 2e-2 would be too tight for the smallest gradients after
-    that depth: 5e-2) with cosine >= 0.999; the loss must agree to 1e-3 relative."""
+    bf16 autocast over fp32 parameters and an fp32 residual stream.  Twelve layers of bf16 rounding separate any two bf16
+    runs of this model, so the bar is a measured one: the model's fp32 run is the ground truth, and every gradient of the
+    HIP run must sit no further from it than the stock-op bf16 run does (see _bf16_against_fp32_truth).  Against each other
+    the two bf16 runs meet the per-tensor bf16 bar (max relative error 2e-2, cosine 0.9999) on all but the few gradients
+    where the stock-op bf16 run is itself further than that from the fp32 truth (the embedding-side biases, 3.8e-2)."""
     cfg = GPTConfig()
     hip, ref = _pair(cfg)
     ids = torch.randint(0, cfg.vocab_size, (16, 1024), generator=torch.Generator().manual_seed(0)).to(DEV)
-    loss, grads = _train_step(hip, ids, autocast=True)
-    loss_ref, grads_ref = _train_step(ref, ids, autocast=True)
-    print(f"config5 loss hip {loss.item():.6f} oracle {loss_ref.item():.6f}")
-    assert abs(loss.item() - loss_ref.item()) <= 1e-3 * abs(loss_ref.item())
-    worst = (0.0, 1.0, "")
-    for name in grads:
-        assert torch.isfinite(grads[name]).all(), name
-        err, cos = rel_err(grads[name], grads_ref[name]), cosine(grads[name], grads_ref[name])
-        if err > worst[0]:
-            worst = (err, cos, name)
-        assert err <= 5e-2 and cos >= 0.999, f"{name}: max relative error {err:.3e}, cosine {cos:.6f}"
-    print(f"config5 worst gradient: {worst[2]} max relative error {worst[0]:.3e} cosine {worst[1]:.6f}")
+    table = _bf16_against_fp32_truth(hip, ref, ids, "config5")
+    at_bar = sum(1 for r in table if r[5] <= 2e-2 and r[6] >= 0.9999)
+    print(f"config5: {at_bar} of {len(table)} gradients meet 2e-2 / 0.9999 hip-bf16 against stock-bf16")
+    for name, e_hip, c_hip, e_stock, c_stock, e_pair, c_pair in table:
+        if e_stock <= 2e-2 and c_stock >= 0.9999:  # where bf16 itself is that close to the truth, so must the pair be
+            assert e_pair <= 2e-2 and c_pair >= 0.9999, f"{name}: hip bf16 against stock bf16 {e_pair:.3e} / {c_pair:.6f}"

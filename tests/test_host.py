@@ -186,3 +186,72 @@ def test_argument_errors_are_reported_not_crashed():
     assert status == 1 and b"bad sizes" in lib.lt_last_error()
     with pytest.raises(RuntimeError, match="lt_status 1"):
         nat.check(status, "lt_ffn_forward")
+
+
+def test_legacy_checkpoint_keys_and_missing_layout_buffers(tmp_path):
+    """A checkpoint in the reference's older naming (the substitutions of reference tests/test_gpt_exact_match.py:51-80),
+    without the `.layout` buffers those checkpoints lacked, written by a module that shares no class with this package,
+    read back with weights_only=True and loaded through load_reference_state_dict."""
+    from lookalike import LookAlikeFFN, LookAlikeLinear, LookAlikeMatrix
+    torch.manual_seed(0)
+    hidden, inter = 64, 128
+    src = LookAlikeFFN(hidden, inter, True, LookAlikeLinear(LookAlikeMatrix(hidden, 2 * inter, 16, 4), 2),
+                       LookAlikeLinear(LookAlikeMatrix(inter, hidden, 16, 4), 2), post_layer_norm=True)
+    legacy = {}
+    for key, value in src.state_dict().items():
+        if key.endswith(".layout"):
+            continue
+        key = "ffn." + key
+        for new, old in ((".matrix.", ".shared_matrix."), (".i2h_proj", ".dense_i2h"), (".h2o_proj", ".dense_h2o"),
+                         ("ffn.pre_layer_norm", "ffn.layer_norm"), (".post_layer_norm", ".sandwich_norm")):
+            key = key.replace(new, old)
+        legacy[key[len("ffn."):]] = value
+    assert "dense_i2h.shared_matrix.weight" in legacy and "sandwich_norm.weight" in legacy and "layer_norm.bias" in legacy
+    path = tmp_path / "legacy.pth"
+    torch.save(legacy, path)
+    state = torch.load(path, weights_only=True)
+    converted = lt.convert_legacy_state_dict({"ffn." + k: v for k, v in state.items()})
+    assert "ffn.i2h_proj.matrix.weight" in converted and "ffn.pre_layer_norm.bias" in converted
+
+    def make():
+        up = lt.GeneralizedLinear(lt.GeneralizedMatrix(hidden, 2 * inter, "pixelfly(16)", lowrank_dim=4), adapter_dim=2)
+        down = lt.GeneralizedLinear(lt.GeneralizedMatrix(inter, hidden, "pixelfly(16)", lowrank_dim=4), adapter_dim=2)
+        return lt.LeanFFN(hidden, inter, gated=True, post_layer_norm=True, layer_norm_eps=1e-5, i2h_proj=up, h2o_proj=down)
+
+    class Wrapper(nn.Module):  # the legacy renames are written for keys inside a model ("...ffn.layer_norm")
+        def __init__(self):
+            super().__init__()
+            self.ffn = make()
+
+    dst = Wrapper()
+    report = lt.load_reference_state_dict(dst, {"ffn." + k: v for k, v in state.items()})
+    assert not report.missing_keys and not report.unexpected_keys
+    for key, value in src.state_dict().items():
+        assert torch.equal(dst.ffn.state_dict()[key], value), key
+    # a checkpoint written for another layout is refused instead of scattering its blocks to the wrong places
+    other = LookAlikeFFN(hidden, inter, True, LookAlikeLinear(LookAlikeMatrix(hidden, 2 * inter, 16, 4, stretch=True), 2),
+                         LookAlikeLinear(LookAlikeMatrix(inter, hidden, 16, 4), 2), post_layer_norm=True)
+    with pytest.raises(ValueError):
+        lt.load_reference_state_dict(make(), other.state_dict())
+    with pytest.raises(RuntimeError):
+        lt.load_reference_state_dict(make(), {k: v for k, v in src.state_dict().items() if "adapter" not in k})
+
+
+def test_native_and_block_list_weight_orders():
+    """native [in, A, block] <-> row-major list of [block, block] sub-matrices, against the oracle's dense expansion"""
+    from oracle import blocksparse as obs
+    torch.manual_seed(1)
+    for out_f, in_f, block, stretch in ((256, 64, 16, False), (64, 256, 16, True), (128, 128, 8, False)):
+        m = lt.GeneralizedMatrix(in_f, out_f, f"pixelfly({block}, stretch={stretch})")
+        w = m.weight.detach()
+        blocks, coords = lt.native_to_block_list(w, m.backward_indices, out_f)
+        dense = obs.sparse_to_dense(w, m.backward_indices.numpy(), out_f)
+        nz = m.layout.nonzero()
+        assert torch.equal(coords, nz)  # row-major order of the layout's active blocks
+        for n, (ob, ib) in enumerate(coords.tolist()):
+            assert torch.equal(blocks[n], dense[ob * block:(ob + 1) * block, ib * block:(ib + 1) * block])
+        assert torch.equal(lt.block_list_to_native(blocks, coords, m.backward_indices), w)
+        perm = torch.randperm(len(blocks))
+        assert torch.equal(lt.block_list_to_native(blocks[perm], coords[perm], m.backward_indices), w)
+    with pytest.raises(ValueError):
+        lt.block_list_to_native(blocks, coords.flip(1), m.backward_indices[:, :1])

@@ -211,3 +211,24 @@ def test_plain_ffn_is_the_textbook_composition():
     o = (o - mu2) / torch.sqrt(var2 + 1e-3) * p.post_ln_weight + p.post_ln_bias
     ref = o * mask / 0.5 + x
     assert torch.allclose(offn.plain_ffn(x, p, mask), ref, rtol=1e-12, atol=1e-12)
+
+
+def test_bf16_rounding_points_are_straight_through_and_representable():
+    """FFNConfig.bf16_rounding: values land on bfloat16's grid (8 significant bits, round to nearest even: known answers),
+    gradients pass unchanged, and with smooth activations the rounded forward stays within bf16 noise of the exact one"""
+    from oracle.ffn import round_bf16_straight_through as rnd
+    t = torch.tensor([1.0, 1.00390625, 1.01171875, -3.0e-5, 257.0, 258.0, 259.0], requires_grad=True)
+    r = rnd(t)
+    # 1 + 2^-8 is a tie between 1 and 1 + 2^-7 -> even (1.0); 1 + 3 * 2^-8 ties to 1 + 2^-6; 257 ties to 256, 259 to 260
+    assert torch.equal(r.detach()[:3], torch.tensor([1.0, 1.0, 1.015625]))
+    assert torch.equal(r.detach()[4:], torch.tensor([256.0, 258.0, 260.0]))
+    assert torch.equal(r.detach(), r.detach().to(torch.bfloat16).float())
+    (g,) = torch.autograd.grad(r.sum(), t)
+    assert torch.equal(g, torch.ones_like(t))
+    gen = torch.Generator().manual_seed(0)
+    x, dy = torch.randn(64, 32, generator=gen), torch.randn(64, 32, generator=gen)
+    exact = offn.make_dense_params(32, 64, gated=True, generator=gen, ln_eps=1e-5)
+    rounded = offn.FFNParams(exact.ln_weight, exact.ln_bias, exact.i2h, exact.h2o,
+                             cfg=offn.FFNConfig(gated=True, ln_eps=1e-5, bf16_rounding=True))
+    y0, y1 = offn.plain_ffn(x, exact), offn.plain_ffn(x, rounded)
+    assert 0 < (y0 - y1).abs().max() / y0.abs().max() < 2e-2
