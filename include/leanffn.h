@@ -148,6 +148,19 @@ int lt_layernorm_backward(int64_t tokens, int32_t hidden, int32_t x_dtype, const
                           const void* residual_grad, void* dx, float* dweight, float* dbias, void* workspace,
                           size_t workspace_bytes, void* stream);
 
+/* lt_layernorm_backward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid allocation).  No counterpart in the reference.  Same arguments and results as
+ * lt_layernorm_backward without the workspace: the partial parameter-gradient rows go to a buffer of
+ * lt_layernorm_backward_static_scratch_bytes() (8 MiB) that the library holds in static device memory, one copy per GPU,
+ * looked up on the first call on each device.  The device that owns `stream` must be the current device.  Rows of a
+ * multiple of 4 elements with 16-byte aligned pointers fit for every tokens / hidden <= 8192; other shapes are refused
+ * with LT_ERR_UNSUPPORTED once tokens * hidden * 8 bytes (tokens capped at 1024) exceed the buffer.  Calls no allocator.
+ * All calls on one GPU share the buffer: calls that overlap in time on the same GPU (different streams) race. */
+size_t lt_layernorm_backward_static_scratch_bytes(void);
+int lt_layernorm_backward_static(int64_t tokens, int32_t hidden, int32_t x_dtype, const void* x, const float* stats,
+                                 const float* weight, int32_t dy_dtype, const void* dy, int32_t dx_dtype,
+                                 const void* residual_grad, void* dx, float* dweight, float* dbias, void* stream);
+
 /* ---- activation alone (for tests of the in-register maths) ------------------------------------------------------------ */
 /* pre [T, 2I or I] -> hid [T, I] */
 int lt_activation_forward(int64_t tokens, int32_t intermediate, int32_t gated, int32_t act, int32_t dtype,

@@ -23,6 +23,7 @@ EXPORTED_SYMBOLS = (
     "lt_linear_backward_workspace_bytes", "lt_linear_forward", "lt_linear_backward",
     "lt_blocksparse_forward", "lt_blocksparse_backward",
     "lt_layernorm_forward", "lt_layernorm_backward_workspace_bytes", "lt_layernorm_backward",
+    "lt_layernorm_backward_static_scratch_bytes", "lt_layernorm_backward_static",
     "lt_activation_forward", "lt_activation_backward", "lt_dropout_mask", "lt_gemm",
     "lt_profile_enable", "lt_profile_reset", "lt_profile_read",
 )
@@ -93,6 +94,10 @@ def _declare(lib):
     lib.lt_layernorm_backward_workspace_bytes.argtypes = [c_int64, c_int32]
     lib.lt_layernorm_backward.argtypes = [c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p,
                                           c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
+    lib.lt_layernorm_backward_static_scratch_bytes.restype = c_size_t
+    lib.lt_layernorm_backward_static_scratch_bytes.argtypes = []
+    lib.lt_layernorm_backward_static.argtypes = [c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p,
+                                                 c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.lt_activation_forward.argtypes = [c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p]
     lib.lt_activation_backward.argtypes = [c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
                                            c_void_p]

@@ -1,5 +1,7 @@
 // HBM-bound kernels of the FFN path: LayerNorm forward / backward with wavefront-shuffle row reductions, column sums for
 // bias / LayerNorm-parameter gradients, stand-alone activation forward / backward, dropout replay and the dropout mask.
+#include <mutex>
+
 #include "lt_internal.h"
 
 namespace {
@@ -702,6 +704,60 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
     LT_LAUNCH_CHECK();
   }
   return LT_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// LayerNorm backward for callers that cannot allocate device memory.  The partial (dweight, dbias) rows live in a
+// file-scope device array instead of a caller workspace.  Each GPU holds its own copy of the array at its own address,
+// looked up once per device; host code only ever uses that looked-up address, never the array's name.
+// ---------------------------------------------------------------------------------------------------------------------
+constexpr size_t LT_LN_STATIC_SCRATCH_BYTES = (size_t)8 << 20;  // 128 row slices x (dweight, dbias) x 8192 columns x 4 bytes
+static __device__ __align__(256) unsigned char scratch[LT_LN_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int LT_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[LT_MAX_DEVICES] = {};
+
+// device address of `scratch` on the device `stream` belongs to, which must be the current device
+int static_scratch_for(hipStream_t stream, void** out) {
+  int current = -1, owner = -1;
+  LT_HIP(hipGetDevice(&current));
+  LT_HIP(hipStreamGetDevice(stream, &owner));
+  LT_REQUIRE(owner == current, LT_ERR_BAD_ARG,
+             "layernorm backward (static scratch): the stream belongs to device %d but device %d is current", owner, current);
+  LT_REQUIRE(current >= 0 && current < LT_MAX_DEVICES, LT_ERR_UNSUPPORTED, "device index %d above %d", current, LT_MAX_DEVICES - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[current]) {
+    void* ptr = nullptr;
+    LT_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    LT_REQUIRE(ptr != nullptr, LT_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch");
+    g_scratch_ptr[current] = ptr;
+  }
+  *out = g_scratch_ptr[current];
+  return LT_OK;
+}
+}  // namespace
+
+extern "C" size_t lt_layernorm_backward_static_scratch_bytes(void) { return LT_LN_STATIC_SCRATCH_BYTES; }
+
+extern "C" int lt_layernorm_backward_static(int64_t tokens, int32_t hidden, int32_t x_dtype, const void* x, const float* stats,
+                                            const float* weight, int32_t dy_dtype, const void* dy, int32_t dx_dtype,
+                                            const void* residual_grad, void* dx, float* dweight, float* dbias,
+                                            void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  for (int d : {x_dtype, dy_dtype, dx_dtype})
+    LT_REQUIRE(d == LT_F32 || d == LT_BF16, LT_ERR_BAD_ARG, "layernorm backward (static scratch): unknown dtype %d", d);
+  void* ptr = nullptr;
+  if (dweight) LT_TRY(static_scratch_for(stream, &ptr));
+  const int status = lt_ln_backward(tokens, hidden, x_dtype, x, stats, weight, dy_dtype, dy, dx_dtype, residual_grad, dx,
+                                    dweight, dbias, ptr, LT_LN_STATIC_SCRATCH_BYTES, stream);
+  if (status == LT_ERR_WORKSPACE)
+    LT_FAIL(LT_ERR_UNSUPPORTED,
+            "layernorm backward (static scratch): tokens=%lld hidden=%d needs more than the %zu-byte static buffer "
+            "(rows of a multiple of 4 elements with 16-byte aligned pointers always fit); use lt_layernorm_backward",
+            (long long)tokens, hidden, LT_LN_STATIC_SCRATCH_BYTES);
+  return status;
 }
 
 // slices of 64 rows (8 per thread), at most 64 of them: 16 x 64 workgroups at 4096 columns, enough to keep every CU's
