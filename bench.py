@@ -79,26 +79,79 @@ def algorithmic_flops(cfg):
     return 3.0 * tokens * fwd
 
 
-def cpu_baseline(torch, hidden, inter, std, sample_tokens, iters):
-    """the oracle's memory-lean autograd.Function (same save-set and recompute schedule as the reference's _LeanFFN) in fp32
-    on the host cores, on the first `sample_tokens` tokens of the workload"""
+def oracle_params_of(torch, ffn, device, dtype):
+    """the module's parameters as the oracle's containers (copies in `dtype` on `device`, requiring grad)"""
     from oracle import ffn as offn
 
-    g = torch.Generator().manual_seed(0)
-    x = torch.randn(sample_tokens, hidden, generator=g)
-    p = offn.make_dense_params(hidden, inter, gated=True, std=std, generator=g, ln_eps=1e-5)
-    for t in p.tensors():
-        t.requires_grad_(True)
-    dy = torch.randn(sample_tokens, hidden, generator=g)
-    x.requires_grad_(True)
+    def leaf(t):
+        return None if t is None else t.detach().to(device=device, dtype=dtype).clone().requires_grad_(True)
+
+    def lin(proj):
+        matrix = getattr(proj, "matrix", None)
+        if matrix is None:
+            return offn.LinearParams(leaf(proj.weight), leaf(proj.bias), out_features=proj.out_features)
+        first, second = proj.get_combined_lowrank_components()
+        fwd, bwd = matrix.forward_indices, matrix.backward_indices
+        return offn.LinearParams(leaf(proj.weight), leaf(proj.bias), leaf(first), leaf(second),
+                                 None if fwd is None else fwd.cpu(), None if bwd is None else bwd.cpu(),
+                                 out_features=proj.out_features)
+
+    return offn.FFNParams(leaf(ffn.pre_layer_norm.weight), leaf(ffn.pre_layer_norm.bias), lin(ffn.i2h_proj),
+                          lin(ffn.h2o_proj),
+                          cfg=offn.FFNConfig(gated=ffn.gated, ln_eps=ffn.pre_layer_norm.eps, residual=ffn.residual))
+
+
+def cpu_baseline(torch, ffn, x, dy, sample_tokens, warmup, iters):
+    """the oracle's memory-lean autograd.Function (same save-set and recompute schedule as the reference's _LeanFFN) in fp32
+    on the host cores, on the first `sample_tokens` tokens of the selected workload (dropout off: it draws no time)"""
+    from oracle import ffn as offn
+
+    hidden = x.shape[-1]
+    p = oracle_params_of(torch, ffn, "cpu", torch.float32)
+    xs = x.detach().reshape(-1, hidden)[:sample_tokens].float().cpu().clone().requires_grad_(True)
+    dys = dy.detach().reshape(-1, hidden)[:sample_tokens].float().cpu()
     times = []
-    for i in range(iters + 1):
+    for i in range(warmup + iters):
         t0 = time.perf_counter()
-        y = offn.lean_ffn(x, p)
-        torch.autograd.grad(y, [x, *p.tensors()], dy)
+        y = offn.lean_ffn(xs, p)
+        torch.autograd.grad(y, [xs, *p.tensors()], dys)
         times.append(time.perf_counter() - t0)
-    best = sorted(times[1:])[len(times[1:]) // 2]
-    return sample_tokens / best, best
+    timed = sorted(times[warmup:])
+    median = timed[len(timed) // 2]
+    return sample_tokens / median, median
+
+
+def reference_activation_memory(torch, ffn, x, dy):
+    """(saved MiB, peak MiB) of one fwd+bwd of the oracle's LeanFFNFunction -- the reference's schedule: keep x and the
+    pre-activation, recompute LayerNorm output and activation in backward -- on the GPU under bf16 autocast with the same
+    weights, input and upstream gradient, measured the way the build's own figures are.  Outside every timed region."""
+    from oracle import ffn as offn
+
+    p = oracle_params_of(torch, ffn, x.device, next(ffn.parameters()).dtype)
+    xr = x.detach().clone().requires_grad_(True)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = offn.lean_ffn(xr, p)
+    torch.cuda.synchronize()
+    saved = (torch.cuda.memory_allocated() - base - y.numel() * y.element_size()) / 2**20
+    torch.autograd.grad(y, [xr, *p.tensors()], dy.to(y.dtype))
+    torch.cuda.synchronize()
+    peak = (torch.cuda.max_memory_allocated() - base) / 2**20
+    return saved, peak
+
+
+def measured_traffic(config):
+    """L2 <-> memory bytes per GEMM launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE summary kept under profiles/ for this
+    configuration (written when that summary is refreshed), with the algorithmic bytes of the same launches; (None, None)
+    when the configuration has no such summary"""
+    path = os.path.join(ROOT, "profiles", f"leanffn_config{config[1:]}_gemm_hbm_traffic.json")
+    if not os.path.exists(path):
+        return None, None
+    with open(path) as f:
+        d = json.load(f)
+    return float(d["bytes_per_gemm_launch"]), float(d["algorithmic_bytes_per_gemm_launch"])
 
 
 def library_gemm_yardstick(torch, cfg, device, iters=10):
@@ -139,6 +192,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing (profiling runs)")
+    ap.add_argument("--no-reference-memory", action="store_true", help="skip the reference-schedule activation memory "
+                    "measurement (the oracle's LeanFFNFunction under bf16 autocast on the GPU; profiling runs)")
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS), help="benchmark configuration (default: the "
                     "headline config 3; the others are reported for reference)")
     ap.add_argument("--yardstick", action="store_true", help="also time torch.matmul (vendor GEMM library, no epilogue) on "
@@ -219,10 +274,10 @@ def main():
                      **({"tflops": fl / (ms * 1e-3) / 1e12} if fl > 0 else {}),
                      **({"gbps": by / (ms * 1e-3) / 1e9} if by > 0 else {})} for name, n, ms, fl, by in kernels]
 
-    # L2 <-> memory bytes per GEMM launch (fetch + write, averaged over the six launches of a step), from the FETCH_SIZE
-    # and WRITE_SIZE counter runs of this command summarised in profiles/leanffn_config3_gemm_hbm_traffic.txt
-    # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration on the dy cast kernel); only measured for config 3
-    traffic = 1.588e9 if args.config == "c3" else None
+    # L2 <-> memory bytes per GEMM launch (fetch + write, averaged over the GEMM launches of a step), from the FETCH_SIZE
+    # and WRITE_SIZE counter runs of this command summarised under profiles/ (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after
+    # calibration on the dy cast kernel, a plain copy of known size)
+    traffic, traffic_algorithmic = measured_traffic(args.config)
 
     result = {
         "metric": METRIC, "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
@@ -234,19 +289,27 @@ def main():
         "peak_activation_mb": peak_mb, "saved_activation_mb": saved_mb,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": traffic,
+                     "traffic_over_algorithmic": (traffic / traffic_algorithmic) if traffic else None,
                      "kernel": "all GEMM launches of a step: " + ", ".join(sorted({k[0] for k in gemm})),
                      "flops_per_launch": gemm_flops / max(gemm_launches, 1),
                      "avg_launch_us": gemm_ms / max(gemm_launches, 1) * 1e3},
         "kernels": kernel_table,
     }
+    if not args.no_reference_memory:
+        ref_saved, ref_peak = reference_activation_memory(torch, ffn, x, dy)
+        result["reference_saved_activation_mb"] = ref_saved
+        result["reference_peak_activation_mb"] = ref_peak
     if not args.no_cpu_baseline:
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
-        sample = min(2048, tokens)  # about 10 s of host work with the warm-up
-        value, sec = cpu_baseline(torch, 4096, 16384, 0.01, sample, iters=3)
+        # bounded sample: about 15 s of host work (8 fwd+bwd) whatever the configuration
+        per_token = flops_per_step / tokens if not cfg["sparse"] else 6.0 * hidden * (
+            (2 * inter if cfg["gated"] else inter) + inter)  # the oracle multiplies the dense expansion of a sparse weight
+        sample = int(min(tokens, max(256, 2048 * 1.208e9 / per_token)))
+        value, sec = cpu_baseline(torch, ffn, x, dy, sample, warmup=3, iters=5)
         result["cpu_baseline"] = {
             "value": value, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"oracle LeanFFNFunction (stock PyTorch fp32, reference save-set) on the first {sample} of {tokens} "
-                      f"tokens of config 3, median of 3 fwd+bwd after 1 warm-up, {sec:.2f} s each"}
+                      f"tokens of {args.config}, median of 5 fwd+bwd after 3 warm-ups, {sec:.2f} s each"}
     if args.yardstick and not cfg["sparse"] and cfg["dtype"] == "bf16":
         result["library_gemm_yardstick"] = library_gemm_yardstick(torch, cfg, device)
     print(json.dumps(result))

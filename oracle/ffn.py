@@ -206,7 +206,10 @@ class LeanFFNFunction(torch.autograd.Function):
     that autograd routes their gradients.
     """
 
+    # custom_fwd / custom_bwd as on the reference's _LeanFFN (ffn.py:146-147,232-233): backward runs under the autocast state
+    # of the forward, so that under torch.autocast(bfloat16) its matmuls take bf16 operands as the forward's did
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, x, keep_mask, params: FFNParams, *param_tensors):
         cfg = params.cfg
         x2d = x.reshape(-1, x.shape[-1])
@@ -229,6 +232,7 @@ class LeanFFNFunction(torch.autograd.Function):
         return out.reshape(x.shape)
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         params: FFNParams = ctx.params
         cfg = params.cfg
