@@ -34,10 +34,21 @@ def _run(cmd):
     return proc.stdout
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
-    """Compile every translation unit (in parallel) and link the shared library; returns its path."""
+TILE_TIMING_LIB_PATH = os.path.join(CSRC, "libleanffn_tile_timing.so")
+
+
+def build(verbose: bool = False, extra_flags=(), tile_timing: bool = False) -> str:
+    """Compile every translation unit (in parallel) and link the shared library; returns its path.
+
+    tile_timing: build the instrumented library instead (csrc/libleanffn_tile_timing.so, -DLT_TILE_TIMING: the copy-based
+    GEMM kernels record per-workgroup phase timestamps; read by lean_transformer_amd/tile_timing.py).  Never loaded by the
+    package itself."""
     hipcc = _hipcc()
-    objects = [os.path.join(CSRC, src.replace(".hip", ".o")) for src in SOURCES]
+    suffix = ".tile_timing.o" if tile_timing else ".o"
+    lib_path = TILE_TIMING_LIB_PATH if tile_timing else LIB_PATH
+    if tile_timing:
+        extra_flags = (*extra_flags, "-DLT_TILE_TIMING")
+    objects = [os.path.join(CSRC, src.replace(".hip", suffix)) for src in SOURCES]
 
     def compile_one(pair):
         src, obj = pair
@@ -47,9 +58,9 @@ def build(verbose: bool = False, extra_flags=()) -> str:
 
     with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, 8, len(SOURCES))) as pool:
         list(pool.map(compile_one, zip(SOURCES, objects)))
-    _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objects, "-o", LIB_PATH])
-    return LIB_PATH
+    _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objects, "-o", lib_path])
+    return lib_path
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, tile_timing="--tile-timing" in sys.argv))

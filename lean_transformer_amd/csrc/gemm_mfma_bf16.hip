@@ -1,6 +1,9 @@
 // Host side of the tiled bf16 GEMMs: which problems the kernels of gemm_mfma_kernels.h take, which kernel a problem goes
 // to, split reductions and their summing passes.  The kernels are instantiated per epilogue kind in gemm_mfma_kind*.hip.
 #include "gemm_mfma_kernels.h"
+#ifdef LT_TILE_TIMING
+int& lt_tile_timing_launch_counter() { static int n = 0; return n; }
+#endif
 
 // defined in gemm_mfma_kind{0,1,2,3}.hip (KIND = EPI_STORE, EPI_ACT_FWD, EPI_ACT_BWD, EPI_OUT)
 int lt_mfma_launch_dense_kind0(const GemmProblem& p, int io_dtype, hipStream_t stream);

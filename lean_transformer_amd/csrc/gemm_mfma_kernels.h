@@ -31,6 +31,31 @@
 
 #include "lt_gemm.h"
 
+// Instrumented build (-DLT_TILE_TIMING, python -m lean_transformer_amd._build --tile-timing; never the product library):
+// thread 0 of every workgroup of the copy-based kernel records the shader clock (s_memtime) when it starts, after the
+// prologue, after 16 k-steps, after the main loop and after the epilogue, and the 100 MHz real-time counter at both ends,
+// 8 words per workgroup, into the buffer whose address the environment variable LT_TILE_TIMING_BUFFER holds; copy-based
+// launch number i of the process writes region i % 6 (4096 workgroups each), i.e. one region per GEMM of an FFN step.
+// lean_transformer_amd/tile_timing.py reads them.
+#ifdef LT_TILE_TIMING
+int& lt_tile_timing_launch_counter();  // one counter for the whole library (defined in gemm_mfma_bf16.hip)
+#define LT_TILE_STAMP(slot)                                                          \
+  do {                                                                               \
+    if (tile_stamps && threadIdx.x == 0) tile_stamps[slot] = __builtin_amdgcn_s_memtime(); \
+  } while (0)
+#define LT_TILE_STAMP_REALTIME(slot)                                                     \
+  do {                                                                                   \
+    if (tile_stamps && threadIdx.x == 0) tile_stamps[slot] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#else
+#define LT_TILE_STAMP(slot) \
+  do {                      \
+  } while (0)
+#define LT_TILE_STAMP_REALTIME(slot) \
+  do {                               \
+  } while (0)
+#endif
+
 namespace {
 
 constexpr int BK = 64;
@@ -639,9 +664,235 @@ static_assert(copies_in_flight(false, false, {}, {}, false, 0) == 16 && copies_i
 constexpr BlockSlots SLOTS_NT_A = {{0, 0}}, SLOTS_NT_B = {{2, 2}}, SLOTS_NN_A = {{0, 2}};
 constexpr bool SPLIT_MN_B = true;
 
+// Epilogue of one wavefront's (FM * 32) x 128 sub-tile of a copy-based kernel: acc[i][j] is the 32 x 32 block at rows
+// m0 + wm * WTM + 32 i, columns n0 + wn * 128 + 32 j of the result (gated forward: blocks 0, 1 gate columns, 2, 3 the
+// matching linear columns).  `stage` is 16 KiB of LDS that belongs to this wavefront alone; tile_rows x tile_cols is the
+// workgroup's tile (for the whole-tile test).  The bias is already in the accumulators.
+template <int FM, int KIND, typename TX, int tile_rows, int tile_cols>
+__device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const GemmProblem& p, float* stage, const int64_t m0,
+                                                  const int64_t n0, const int wm, const int wn, const bool gated) {
+  constexpr int FN = 4, WTN = 128, WTM = FM * 32;
+  // the lane index is formed anew (two v_mbcnt) rather than kept in a register across the main loop
+  const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  // ---- epilogue.  The accumulators of a 32 x 32 block sit column-per-lane (register r = row 8 * (r / 4) + 4 * (lane / 32)
+  //      + r % 4, column lane % 32).  Each wavefront transposes one 32-row strip of its sub-tile at a time through an LDS
+  //      buffer of its own (32 x 128 floats = 16 KiB, the size of the smallest buffer) and reads it back row-major, 8
+  //      consecutive columns per lane, so that the fused epilogue reads and writes HBM in 16-byte pieces of contiguous rows.
+  //      Staged column c of row r sits at c ^ 32 when bit 2 of r is set: the two half-waves of a transposing write (rows
+  //      r and r + 4, same columns) then hit different banks without padding the rows.
+  EpiParams epi = p.epi;
+  epi.bias = nullptr;  // already in the accumulators
+  if (KIND == EPI_STORE && p.ksplit > 1) epi.out = reinterpret_cast<float*>(epi.out) + (int64_t)blockIdx.y * p.split_stride;
+  auto staged = [&](int row, int col) -> float* { return &stage[row * WTN + (col ^ (((row >> 2) & 1) << 5))]; };
+  const bool pair = (KIND == EPI_ACT_FWD) && gated;
+  float colsum[16];  // EPI_ACT_BWD: column sums of this lane's 8 (+ 8) dpre columns over the rows it writes
+#pragma unroll
+  for (int e = 0; e < 16; e++) colsum[e] = 0.f;
+  // accumulators of strip I -> this wavefront's staging buffer
+  auto stage_strip = [&](auto I) {
+    constexpr int i = decltype(I)::value;
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) *staged(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), j * 32 + (lane & 31)) = acc[i][j][r];
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto for_each_strip = [&](auto&& strip) { lt_static_for<FM>(strip); };
+  auto generic_strip = [&](auto I) {
+    constexpr int i = decltype(I)::value;
+    stage_strip(I);
+    const int64_t mrow0 = m0 + wm * WTM + i * 32;
+    if (pair) {
+      // columns [0, WTN/2) of the sub-tile are gate columns, [WTN/2, WTN) the matching linear columns
+      constexpr int LANES_PER_ROW = WTN / 2 / 8, ROWS_PER_IT = 64 / LANES_PER_ROW;
+      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+        const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW, c = (lane % LANES_PER_ROW) * 8;
+        const int64_t m = mrow0 + row;
+        float vg[8], vl[8];
+        const float* sg = staged(row, c);
+        const float* sl = staged(row, WTN / 2 + c);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          vg[e] = sg[e];
+          vl[e] = sl[e];
+        }
+        const int64_t n = n0 + wn * (WTN / 2) + c;
+        if (m < p.M && n < p.N) epi_act_fwd_gated8(epi, m, n, vg, vl);
+      }
+    } else {
+      constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+      const int c = (lane % LANES_PER_ROW) * 8;
+      const int64_t n = n0 + wn * WTN + c;
+      const bool in_n = n < p.N;  // N is a multiple of 8: the lane's 8 columns are all inside or all outside
+      const int64_t mlane = mrow0 + lane / LANES_PER_ROW;  // this lane's row in iteration 0
+      // global reads of the epilogue run two iterations ahead of their use
+      EpiLoad l0 = epi_load8<KIND, TX>(epi, mlane, n, in_n && mlane < p.M);
+      EpiLoad l1 = epi_load8<KIND, TX>(epi, mlane + ROWS_PER_IT, n, in_n && mlane + ROWS_PER_IT < p.M);
+      for (int it = 0; it < NIT; it++) {
+        const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
+        const int64_t m = mrow0 + row;
+        const int64_t m2 = m + 2 * ROWS_PER_IT;
+        const EpiLoad l2 = epi_load8<KIND, TX>(epi, m2, n, in_n && it + 2 < NIT && m2 < p.M);
+        float v[8];
+        const float* sv = staged(row, c);
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = sv[e];
+        if (in_n && m < p.M) {
+          if constexpr (KIND == EPI_STORE) epi_store8(epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(epi, m, n, v);
+          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(epi, m, n, v, l0, colsum);
+          else epi_out8_loaded<TX>(epi, m, n, v, l0);
+        }
+        l0 = l1;
+        l1 = l2;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  // One lane's share of the staged strip: NIT rows x 8 columns starting at column c, fetched with 16-byte LDS reads that all
+  // go out before the first value is used, so that a strip exposes the LDS latency once and not once per row (one wavefront
+  // per SIMD: nobody else would hide it).  The registers come from the accumulators of the strip just staged.
+  auto read_staged_rows = [&](auto nit_c, auto rows_per_it_c, int lanes_per_row, int c, float (&v)[decltype(nit_c)::value][8]) {
+    constexpr int NIT_ = decltype(nit_c)::value, RPI = decltype(rows_per_it_c)::value;
+    f32x4 raw[NIT_][2];
+#pragma unroll
+    for (int it = 0; it < NIT_; it++) {
+      const float* sv = staged(it * RPI + lane / lanes_per_row, c);
+      raw[it][0] = *reinterpret_cast<const f32x4*>(sv);
+      raw[it][1] = *reinterpret_cast<const f32x4*>(sv + 4);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT_; it++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) v[it][e] = raw[it][e >> 2][e & 3];
+  };
+  // EPI_ACT_BWD, the usual case (whole tile in range, tanh GELU, h wanted): straight-line strips.  The pre-activation reads
+  // of ACT_WINDOW rows are in flight at any time -- the first window goes out before the strip is staged -- and, with no
+  // branches in between, each row waits only for its own reads.
+  constexpr int ACT_WINDOW = 3;
+  auto act_bwd_strip = [&](auto I, auto G) {
+    constexpr int i = decltype(I)::value;
+    constexpr bool GATED = decltype(G)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * WTN + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    EpiLoad win[ACT_WINDOW];
+#pragma unroll
+    for (int it = 0; it < ACT_WINDOW; it++) win[it] = epi_load_pre8<GATED>(epi, mlane + it * ROWS_PER_IT, n);
+    stage_strip(I);
+    float v[NIT][8];
+    read_staged_rows(std::integral_constant<int, NIT>{}, std::integral_constant<int, ROWS_PER_IT>{}, LANES_PER_ROW, c, v);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      epi_act_bwd8_gelu<GATED>(epi, mlane + it * ROWS_PER_IT, n, v[it], win[it % ACT_WINDOW], colsum);
+      if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_pre8<GATED>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  // The other kinds, same idea: whole tile in range, tanh GELU, no dropout, residual present.
+  const bool whole_tile = m0 + tile_rows <= p.M && n0 + (gated ? tile_cols / 2 : tile_cols) <= p.N;
+  auto act_fwd_strip = [&](auto I, auto G) {
+    constexpr int i = decltype(I)::value;
+    constexpr bool GATED = decltype(G)::value;
+    constexpr int LANES_PER_ROW = (GATED ? WTN / 2 : WTN) / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * (GATED ? WTN / 2 : WTN) + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    stage_strip(I);
+    float v0[NIT][8], v1[GATED ? NIT : 1][8];
+    read_staged_rows(std::integral_constant<int, NIT>{}, std::integral_constant<int, ROWS_PER_IT>{}, LANES_PER_ROW, c, v0);
+    if constexpr (GATED)
+      read_staged_rows(std::integral_constant<int, NIT>{}, std::integral_constant<int, ROWS_PER_IT>{}, LANES_PER_ROW, WTN / 2 + c, v1);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) epi_act_fwd8_gelu<GATED>(epi, mlane + it * ROWS_PER_IT, n, v0[it], v1[GATED ? it : 0]);
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto store_strip = [&](auto I, auto out_type) {
+    using TO = decltype(out_type);
+    constexpr int i = decltype(I)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * WTN + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    stage_strip(I);
+    float v[NIT][8];
+    read_staged_rows(std::integral_constant<int, NIT>{}, std::integral_constant<int, ROWS_PER_IT>{}, LANES_PER_ROW, c, v);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) epi_store8_plain<TO>(epi, mlane + it * ROWS_PER_IT, n, v[it]);
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto out_strip = [&](auto I, auto D) {
+    constexpr bool DROPOUT = decltype(D)::value;
+    constexpr int i = decltype(I)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int64_t n = n0 + wn * WTN + c;
+    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
+    EpiLoad win[ACT_WINDOW];
+#pragma unroll
+    for (int it = 0; it < ACT_WINDOW; it++) win[it] = epi_load_x8<TX>(epi, mlane + it * ROWS_PER_IT, n);
+    stage_strip(I);
+    float v[NIT][8];
+    read_staged_rows(std::integral_constant<int, NIT>{}, std::integral_constant<int, ROWS_PER_IT>{}, LANES_PER_ROW, c, v);
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      epi_out8_residual<TX, DROPOUT>(epi, mlane + it * ROWS_PER_IT, n, v[it], win[it % ACT_WINDOW]);
+      if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_x8<TX>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  if constexpr (KIND == EPI_ACT_BWD) {
+    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED && epi.hid != nullptr;
+    if (straight && epi.gated) for_each_strip([&](auto I) { act_bwd_strip(I, std::true_type{}); });
+    else if (straight) for_each_strip([&](auto I) { act_bwd_strip(I, std::false_type{}); });
+    else for_each_strip(generic_strip);
+  } else if constexpr (KIND == EPI_ACT_FWD) {
+    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED;
+    if (straight && pair) for_each_strip([&](auto I) { act_fwd_strip(I, std::true_type{}); });
+    else if (straight) for_each_strip([&](auto I) { act_fwd_strip(I, std::false_type{}); });
+    else for_each_strip(generic_strip);
+  } else if constexpr (KIND == EPI_STORE) {
+    if (whole_tile && epi.out_dtype == LT_F32) for_each_strip([&](auto I) { store_strip(I, float{}); });
+    else if (whole_tile) for_each_strip([&](auto I) { store_strip(I, bf16{}); });
+    else for_each_strip(generic_strip);
+  } else {
+    if (whole_tile && epi.x && epi.drop.p == 0.f) {
+      for_each_strip([&](auto I) { out_strip(I, std::false_type{}); });
+    } else if (whole_tile && epi.x) {
+      for_each_strip([&](auto I) { out_strip(I, std::true_type{}); });
+    } else {
+      for_each_strip(generic_strip);
+    }
+  }
+  if constexpr (KIND == EPI_ACT_BWD) {
+    if (epi.colsum) {
+      // lanes l, l + 16, l + 32, l + 48 hold the same columns for different rows of the wavefront's WTM-row sub-tile
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        colsum[e] += __shfl_xor(colsum[e], 16);
+        colsum[e] += __shfl_xor(colsum[e], 32);
+      }
+      // a sub-tile wholly past the last row has no partial row: the caller sizes the buffer for ceil(M / 128) of them
+      if (lane < 16 && n0 + wn * WTN + lane * 8 < p.N && m0 + wm * WTM < p.M) {
+        float* dst = epi.colsum + ((m0 + wm * WTM) / WTM) * epi.ld_pre + n0 + wn * WTN + lane * 8;
+        float lo[8], hi[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          lo[e] = colsum[e];
+          hi[e] = colsum[8 + e];
+        }
+        store8(dst, lo);
+        if (epi.gated) store8(dst + epi.inter, hi);
+      }
+    }
+  }
+}
+
 template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
+  constexpr int HALF = 4;  // copy instructions per wavefront for a mn-major k-step or half a k-major block
   constexpr int KM_ELEMS = 256 * 64, MN_ELEMS = DK * 256;
   // k-major operands use the two d buffers, mn-major ones the four s tiles; the unused set is never referenced and takes
   // no LDS
@@ -662,6 +913,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const bool gated = (KIND == EPI_ACT_FWD) && p.epi.gated;
+#ifdef LT_TILE_TIMING
+  // (a dense problem has no use for the block-sparse walk's second activation pointer: the timing buffer rides there)
+  unsigned long long* const tile_stamps =
+      p.sp.act2 ? reinterpret_cast<unsigned long long*>(const_cast<void*>(p.sp.act2)) + (size_t)blockIdx.x * 8 : nullptr;
+#endif
+  LT_TILE_STAMP(0);
+  LT_TILE_STAMP_REALTIME(4);
 
   int pid = blockIdx.x;
   const int num_pid = tiles_m * tiles_n;
@@ -807,9 +1065,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);
   // LDS reads of a half-step spread over this many of its 16 matrix instructions: evenly over all of them, except for the
   // mixed layout, which measured 2 % faster with the reads done by the twelfth
-  constexpr int READ_SPAN = (A_KM && !B_KM) ? 12 : 16;
-  constexpr int N_MN = (A_KM ? 0 : 4) + (B_KM ? 0 : 4);  // copy instructions per k-step for the mn-major operands
-  constexpr int N_KM = (A_KM ? 8 : 0) + (B_KM ? 8 : 0);  // copy instructions per block for the k-major operands
+  constexpr int READ_SPAN = (A_KM && !B_KM) ? FM * FN * 3 / 4 : FM * FN;
+  constexpr int N_MN = (A_KM ? 0 : HALF) + (B_KM ? 0 : HALF);  // copy instructions per k-step for the mn-major operands
+  constexpr int N_KM = (A_KM ? 2 * HALF : 0) + (B_KM ? 2 * HALF : 0);  // copy instructions per block for the k-major operands
 
   bf16x8 af[2][FM], bfr[2][FN];  // [0]: first 16 k of the current k-step, [1]: second 16 k
 
@@ -825,8 +1083,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   constexpr BlockSlots SA = B_KM ? SLOTS_NT_A : SLOTS_NN_A, SB = SLOTS_NT_B;
   constexpr bool B_SPLIT = !B_KM && !A_KM && SPLIT_MN_B;
   using J0 = std::integral_constant<int, 0>;
-  using J4 = std::integral_constant<int, 4>;
-  using J8 = std::integral_constant<int, 8>;
+  using J4 = std::integral_constant<int, HALF>;      // named for the four-wavefront case: half a k-major block,
+  using J8 = std::integral_constant<int, 2 * HALF>;  // a whole one
   // the halves of the k-major blocks assigned to `slot`, for the block that starts at k-step t, into position I
   auto copy_block_halves = [&](auto steady, auto slot, auto I, int t) {
     constexpr int SLOT = decltype(slot)::value;
@@ -836,8 +1094,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     if constexpr (B_KM && SB.half[1] == SLOT) copy_b(steady, I, t, J4{}, J8{});
   };
   auto slot_copies = [&](int slot) constexpr {
-    return (A_KM ? 4 * ((SA.half[0] == slot) + (SA.half[1] == slot)) : 0) +
-           (B_KM ? 4 * ((SB.half[0] == slot) + (SB.half[1] == slot)) : 0);
+    return (A_KM ? HALF * ((SA.half[0] == slot) + (SA.half[1] == slot)) : 0) +
+           (B_KM ? HALF * ((SB.half[0] == slot) + (SB.half[1] == slot)) : 0);
   };
   // LDS reads in flight at the barrier of k-step t are the second 16 k of that k-step (position i).  Copies issued before
   // the next barrier that overwrite that buffer: mn-major copies of the next first half (the ring tile of k-step t), and
@@ -858,7 +1116,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
         copy_block_halves(steady, std::integral_constant<int, 1>{}, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
     }
     mfma_half(af[0], bfr[0]);
-    constexpr int COPIES = (A_KM ? 0 : 4) + ((B_KM || B_SPLIT) ? 0 : 4) + ((i & 1) == 0 ? slot_copies(1) : 0);
+    constexpr int COPIES = (A_KM ? 0 : HALF) + ((B_KM || B_SPLIT) ? 0 : HALF) + ((i & 1) == 0 ? slot_copies(1) : 0);
     SchedInterleave3<FRAG_READS, COPIES, FM * FN, READ_SPAN>::run();
   };
   auto second_half = [&](auto steady, auto I, int t) {
@@ -882,7 +1140,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
         copy_block_halves(steady, std::integral_constant<int, 2>{}, std::integral_constant<int, (i + 2) & 3>{}, t + 2);
     }
     mfma_half(af[1], bfr[1]);
-    constexpr int COPIES = (B_SPLIT ? 4 : 0) + (N_KM > 0 ? slot_copies((i & 1) ? 0 : 2) : 0);
+    constexpr int COPIES = (B_SPLIT ? HALF : 0) + (N_KM > 0 ? slot_copies((i & 1) ? 0 : 2) : 0);
     SchedInterleave3<FRAG_READS, COPIES, FM * FN, READ_SPAN>::run();
   };
   using Steady = std::integral_constant<bool, true>;
@@ -908,6 +1166,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     if constexpr (N_KM > 0) copy_block_halves(Ragged{}, std::integral_constant<int, 0>{}, P2{}, 2);
   }
   wait_copies_and_barrier<0>();
+  LT_TILE_STAMP(1);
   load_frags(P0{}, 0, af[0], bfr[0]);
   first_half(Ragged{}, P0{}, 0);
 
@@ -919,6 +1178,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     const int bound = (ca.seg == 0 && p.nseg > 1) ? kt_seg0 : kt_total;
     if (ca.seg == cb.seg) {
       for (; kt + 7 < bound; kt += 4) {
+#ifdef LT_TILE_TIMING
+        if (kt == 16) LT_TILE_STAMP(7);
+#endif
         second_half(Steady{}, P0{}, kt);
         first_half(Steady{}, P1{}, kt + 1);
         second_half(Steady{}, P1{}, kt + 1);
@@ -939,235 +1201,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     if (kt >= kt_total) break;
   }
   __syncthreads();  // every wavefront is done with the buffers: they become epilogue staging space
+  LT_TILE_STAMP(2);
 
-  // ---- epilogue.  The accumulators of a 32 x 32 block sit column-per-lane (register r = row 8 * (r / 4) + 4 * (lane / 32)
-  //      + r % 4, column lane % 32).  Each wavefront transposes one 32-row strip of its sub-tile at a time through an LDS
-  //      buffer of its own (32 x 128 floats = 16 KiB, the size of the smallest buffer) and reads it back row-major, 8
-  //      consecutive columns per lane, so that the fused epilogue reads and writes HBM in 16-byte pieces of contiguous rows.
-  //      Staged column c of row r sits at c ^ 32 when bit 2 of r is set: the two half-waves of a transposing write (rows
-  //      r and r + 4, same columns) then hit different banks without padding the rows.
-  EpiParams epi = p.epi;
-  epi.bias = nullptr;  // already in the accumulators
-  if (KIND == EPI_STORE && p.ksplit > 1) epi.out = reinterpret_cast<float*>(epi.out) + (int64_t)blockIdx.y * p.split_stride;
-  float* stage = reinterpret_cast<float*>(wave == 0   ? (A_KM ? a_d0 : a_s0)
-                                          : wave == 1 ? (A_KM ? a_d1 : a_s1)
-                                          : wave == 2 ? (B_KM ? b_d0 : b_s0)
-                                                      : (B_KM ? b_d1 : b_s1));
+  // 16 KiB of staging space per wavefront: the first two buffers of each operand
+  bf16* const stage_buf = wave == 0 ? (A_KM ? a_d0 : a_s0) : wave == 1 ? (A_KM ? a_d1 : a_s1) : wave == 2 ? (B_KM ? b_d0 : b_s0) : (B_KM ? b_d1 : b_s1);
+  dma_tile_epilogue<FM, KIND, TX, BM, BN>(acc, p, reinterpret_cast<float*>(stage_buf), m0, n0, wm, wn, gated);
+  LT_TILE_STAMP(3);
+  LT_TILE_STAMP_REALTIME(5);
   static_assert(32 * WTN * 4 <= MN_ELEMS * 2, "a 32-row strip must fit the smallest buffer");
-  auto staged = [&](int row, int col) -> float* { return &stage[row * WTN + (col ^ (((row >> 2) & 1) << 5))]; };
-  const bool pair = (KIND == EPI_ACT_FWD) && gated;
-  float colsum[16];  // EPI_ACT_BWD: column sums of this lane's 8 (+ 8) dpre columns over the rows it writes
-#pragma unroll
-  for (int e = 0; e < 16; e++) colsum[e] = 0.f;
-  // accumulators of strip I -> this wavefront's staging buffer
-  auto stage_strip = [&](auto I) {
-    constexpr int i = decltype(I)::value;
-#pragma unroll
-    for (int j = 0; j < FN; j++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) *staged(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), j * 32 + (lane & 31)) = acc[i][j][r];
-    __builtin_amdgcn_wave_barrier();
-  };
-  auto for_each_strip = [&](auto&& strip) {
-    static_assert(FM == 4, "four 32-row strips per wavefront");
-    strip(std::integral_constant<int, 0>{});
-    strip(std::integral_constant<int, 1>{});
-    strip(std::integral_constant<int, 2>{});
-    strip(std::integral_constant<int, 3>{});
-  };
-  auto generic_strip = [&](auto I) {
-    constexpr int i = decltype(I)::value;
-    stage_strip(I);
-    const int64_t mrow0 = m0 + wm * WTM + i * 32;
-    if (pair) {
-      // columns [0, WTN/2) of the sub-tile are gate columns, [WTN/2, WTN) the matching linear columns
-      constexpr int LANES_PER_ROW = WTN / 2 / 8, ROWS_PER_IT = 64 / LANES_PER_ROW;
-      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
-        const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW, c = (lane % LANES_PER_ROW) * 8;
-        const int64_t m = mrow0 + row;
-        float vg[8], vl[8];
-        const float* sg = staged(row, c);
-        const float* sl = staged(row, WTN / 2 + c);
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-          vg[e] = sg[e];
-          vl[e] = sl[e];
-        }
-        const int64_t n = n0 + wn * (WTN / 2) + c;
-        if (m < p.M && n < p.N) epi_act_fwd_gated8(epi, m, n, vg, vl);
-      }
-    } else {
-      constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
-      const int c = (lane % LANES_PER_ROW) * 8;
-      const int64_t n = n0 + wn * WTN + c;
-      const bool in_n = n < p.N;  // N is a multiple of 8: the lane's 8 columns are all inside or all outside
-      const int64_t mlane = mrow0 + lane / LANES_PER_ROW;  // this lane's row in iteration 0
-      // global reads of the epilogue run two iterations ahead of their use
-      EpiLoad l0 = epi_load8<KIND, TX>(epi, mlane, n, in_n && mlane < p.M);
-      EpiLoad l1 = epi_load8<KIND, TX>(epi, mlane + ROWS_PER_IT, n, in_n && mlane + ROWS_PER_IT < p.M);
-      for (int it = 0; it < NIT; it++) {
-        const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
-        const int64_t m = mrow0 + row;
-        const int64_t m2 = m + 2 * ROWS_PER_IT;
-        const EpiLoad l2 = epi_load8<KIND, TX>(epi, m2, n, in_n && it + 2 < NIT && m2 < p.M);
-        float v[8];
-        const float* sv = staged(row, c);
-#pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = sv[e];
-        if (in_n && m < p.M) {
-          if constexpr (KIND == EPI_STORE) epi_store8(epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_FWD) epi_act_fwd8(epi, m, n, v);
-          else if constexpr (KIND == EPI_ACT_BWD) epi_act_bwd8_loaded(epi, m, n, v, l0, colsum);
-          else epi_out8_loaded<TX>(epi, m, n, v, l0);
-        }
-        l0 = l1;
-        l1 = l2;
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-  };
-  // EPI_ACT_BWD, the usual case (whole tile in range, tanh GELU, h wanted): straight-line strips.  The pre-activation reads
-  // of ACT_WINDOW rows are in flight at any time -- the first window goes out before the strip is staged -- and, with no
-  // branches in between, each row waits only for its own reads.
-  constexpr int ACT_WINDOW = 3;
-  auto act_bwd_strip = [&](auto I, auto G) {
-    constexpr int i = decltype(I)::value;
-    constexpr bool GATED = decltype(G)::value;
-    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
-    const int c = (lane % LANES_PER_ROW) * 8;
-    const int64_t n = n0 + wn * WTN + c;
-    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
-    EpiLoad win[ACT_WINDOW];
-#pragma unroll
-    for (int it = 0; it < ACT_WINDOW; it++) win[it] = epi_load_pre8<GATED>(epi, mlane + it * ROWS_PER_IT, n);
-    stage_strip(I);
-#pragma unroll
-    for (int it = 0; it < NIT; it++) {
-      const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
-      float v[8];
-      const float* sv = staged(row, c);
-#pragma unroll
-      for (int e = 0; e < 8; e++) v[e] = sv[e];
-      epi_act_bwd8_gelu<GATED>(epi, mlane + it * ROWS_PER_IT, n, v, win[it % ACT_WINDOW], colsum);
-      if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_pre8<GATED>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
-    }
-    __builtin_amdgcn_wave_barrier();
-  };
-  // The other kinds, same idea: whole tile in range, tanh GELU, no dropout, residual present.
-  const bool whole_tile = m0 + BM <= p.M && n0 + (gated ? BN / 2 : BN) <= p.N;
-  auto act_fwd_strip = [&](auto I, auto G) {
-    constexpr int i = decltype(I)::value;
-    constexpr bool GATED = decltype(G)::value;
-    constexpr int LANES_PER_ROW = (GATED ? WTN / 2 : WTN) / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
-    const int c = (lane % LANES_PER_ROW) * 8;
-    const int64_t n = n0 + wn * (GATED ? WTN / 2 : WTN) + c;
-    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
-    stage_strip(I);
-#pragma unroll
-    for (int it = 0; it < NIT; it++) {
-      const int row = it * ROWS_PER_IT + lane / LANES_PER_ROW;
-      float v0[8], v1[8];
-      const float* s0 = staged(row, c);
-      const float* s1 = staged(row, GATED ? WTN / 2 + c : c);
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        v0[e] = s0[e];
-        v1[e] = s1[e];
-      }
-      epi_act_fwd8_gelu<GATED>(epi, mlane + it * ROWS_PER_IT, n, v0, v1);
-    }
-    __builtin_amdgcn_wave_barrier();
-  };
-  auto store_strip = [&](auto I, auto out_type) {
-    using TO = decltype(out_type);
-    constexpr int i = decltype(I)::value;
-    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
-    const int c = (lane % LANES_PER_ROW) * 8;
-    const int64_t n = n0 + wn * WTN + c;
-    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
-    stage_strip(I);
-#pragma unroll
-    for (int it = 0; it < NIT; it++) {
-      float v[8];
-      const float* sv = staged(it * ROWS_PER_IT + lane / LANES_PER_ROW, c);
-#pragma unroll
-      for (int e = 0; e < 8; e++) v[e] = sv[e];
-      epi_store8_plain<TO>(epi, mlane + it * ROWS_PER_IT, n, v);
-    }
-    __builtin_amdgcn_wave_barrier();
-  };
-  auto out_strip = [&](auto I, auto D) {
-    constexpr bool DROPOUT = decltype(D)::value;
-    constexpr int i = decltype(I)::value;
-    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
-    const int c = (lane % LANES_PER_ROW) * 8;
-    const int64_t n = n0 + wn * WTN + c;
-    const int64_t mlane = m0 + wm * WTM + i * 32 + lane / LANES_PER_ROW;
-    EpiLoad win[ACT_WINDOW];
-#pragma unroll
-    for (int it = 0; it < ACT_WINDOW; it++) win[it] = epi_load_x8<TX>(epi, mlane + it * ROWS_PER_IT, n);
-    stage_strip(I);
-#pragma unroll
-    for (int it = 0; it < NIT; it++) {
-      float v[8];
-      const float* sv = staged(it * ROWS_PER_IT + lane / LANES_PER_ROW, c);
-#pragma unroll
-      for (int e = 0; e < 8; e++) v[e] = sv[e];
-      epi_out8_residual<TX, DROPOUT>(epi, mlane + it * ROWS_PER_IT, n, v, win[it % ACT_WINDOW]);
-      if (it + ACT_WINDOW < NIT) win[it % ACT_WINDOW] = epi_load_x8<TX>(epi, mlane + (it + ACT_WINDOW) * ROWS_PER_IT, n);
-    }
-    __builtin_amdgcn_wave_barrier();
-  };
-  if constexpr (KIND == EPI_ACT_BWD) {
-    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED && epi.hid != nullptr;
-    if (straight && epi.gated) for_each_strip([&](auto I) { act_bwd_strip(I, std::true_type{}); });
-    else if (straight) for_each_strip([&](auto I) { act_bwd_strip(I, std::false_type{}); });
-    else for_each_strip(generic_strip);
-  } else if constexpr (KIND == EPI_ACT_FWD) {
-    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED;
-    if (straight && pair) for_each_strip([&](auto I) { act_fwd_strip(I, std::true_type{}); });
-    else if (straight) for_each_strip([&](auto I) { act_fwd_strip(I, std::false_type{}); });
-    else for_each_strip(generic_strip);
-  } else if constexpr (KIND == EPI_STORE) {
-    if (whole_tile && epi.out_dtype == LT_F32) for_each_strip([&](auto I) { store_strip(I, float{}); });
-    else if (whole_tile) for_each_strip([&](auto I) { store_strip(I, bf16{}); });
-    else for_each_strip(generic_strip);
-  } else {
-    if (whole_tile && epi.x && epi.drop.p == 0.f) {
-      for_each_strip([&](auto I) { out_strip(I, std::false_type{}); });
-    } else if (whole_tile && epi.x) {
-      for_each_strip([&](auto I) { out_strip(I, std::true_type{}); });
-    } else {
-      for_each_strip(generic_strip);
-    }
-  }
-  if constexpr (KIND == EPI_ACT_BWD) {
-    if (epi.colsum) {
-      // lanes l, l + 16, l + 32, l + 48 hold the same columns for different rows of the wavefront's 128-row sub-tile
-#pragma unroll
-      for (int e = 0; e < 16; e++) {
-        colsum[e] += __shfl_xor(colsum[e], 16);
-        colsum[e] += __shfl_xor(colsum[e], 32);
-      }
-      // a sub-tile wholly past the last row has no partial row: the caller sizes the buffer for ceil(M / 128) of them
-      if (lane < 16 && n0 + wn * WTN + lane * 8 < p.N && m0 + wm * WTM < p.M) {
-        float* dst = epi.colsum + ((m0 + wm * WTM) / 128) * epi.ld_pre + n0 + wn * WTN + lane * 8;
-        float lo[8], hi[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-          lo[e] = colsum[e];
-          hi[e] = colsum[8 + e];
-        }
-        store8(dst, lo);
-        if (epi.gated) store8(dst + epi.inter, hi);
-      }
-    }
-  }
 }
 
 template <bool A_KM, bool B_KM, int KIND>
 int launch_dma(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
   GemmProblem p = problem;
+#ifdef LT_TILE_TIMING
+  if (const char* e = getenv("LT_TILE_TIMING_BUFFER"))
+    p.sp.act2 = (const void*)(strtoull(e, nullptr, 0) + (size_t)(lt_tile_timing_launch_counter()++ % 6) * 4096 * 64);
+#endif
   // k-walk stagger: on unless the caller chose (15: off)
   if (p.krot == 0) p.krot = (A_KM && B_KM) ? 2 : 0;
   else if (p.krot == 15) p.krot = 0;
