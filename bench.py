@@ -186,6 +186,41 @@ def library_gemm_yardstick(torch, cfg, device, iters=10):
     return out
 
 
+def operand_path_yardstick(torch, nat, cfg, device, iters=10):
+    """The library's own plain-store GEMM (lt_gemm) on the up-projection and dW2 shapes with its two operand paths: tiles
+    copied HBM -> LDS without passing through registers (the product path) and tiles staged through registers (the only
+    place where a LayerNorm or an activation could be applied to an operand on its way in).  What fusing LayerNorm into the
+    up-projection's prologue, or recomputing the activation in the weight-gradient GEMM's prologue, would cost in GEMM time
+    before any of the extra arithmetic."""
+    tokens, hidden, inter = cfg["batch"] * cfg["seq"], cfg["hidden"], cfg["inter"]
+    n1 = 2 * inter if cfg["gated"] else inter
+    lib = nat.lib()
+    out = {}
+    for name, (m, n, k, a_km, b_km) in {"up": (tokens, n1, hidden, 1, 1), "dW2": (hidden, inter, tokens, 0, 0)}.items():
+        a = (torch.randn(m * k, device=device) * 0.5).to(torch.bfloat16)
+        b = (torch.randn(n * k, device=device) * 0.02).to(torch.bfloat16)
+        c = torch.empty(m, n, dtype=torch.bfloat16, device=device)
+        row = {"m": m, "n": n, "k": k}
+        for label, force in (("copied_to_lds", 0), ("staged_through_registers", 2)):
+            def run():
+                nat.check(lib.lt_gemm(1, m, n, k, a.data_ptr(), a_km, b.data_ptr(), b_km, 1, c.data_ptr(), force,
+                                      torch.cuda.current_stream().cuda_stream), "lt_gemm")
+            for _ in range(3):
+                run()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record()
+            for _ in range(iters):
+                run()
+            stop.record()
+            torch.cuda.synchronize()
+            us = start.elapsed_time(stop) / iters * 1e3
+            row[label] = {"avg_us": us, "tflops": 2.0 * m * n * k / us / 1e6}
+        out[name] = row
+        del a, b, c
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -312,6 +347,7 @@ def main():
                       f"tokens of {args.config}, median of 5 fwd+bwd after 3 warm-ups, {sec:.2f} s each"}
     if args.yardstick and not cfg["sparse"] and cfg["dtype"] == "bf16":
         result["library_gemm_yardstick"] = library_gemm_yardstick(torch, cfg, device)
+        result["operand_path_yardstick"] = operand_path_yardstick(torch, nat, cfg, device)
     print(json.dumps(result))
 
 
