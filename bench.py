@@ -330,7 +330,18 @@ def main():
                      "avg_launch_us": gemm_ms / max(gemm_launches, 1) * 1e3},
         "kernels": kernel_table,
     }
-    if not args.no_reference_memory:
+    if cfg["sparse"] and traffic:
+        # The block-sparse configuration is bound by memory traffic (its GEMM launches move 5 TB/s through the L2 boundary with
+        # the matrix cores a quarter busy): priced against HBM with the launches' algorithmic bytes (every operand and result
+        # once, from the same counter summary) over their measured duration.
+        avg_launch_s = gemm_ms / max(gemm_launches, 1) * 1e-3
+        result["roofline"].update({"bound": "hbm", "achieved": traffic_algorithmic / avg_launch_s / 1e9, "peak": 8000.0,
+                                   "unit": "GB/s", "frac": traffic_algorithmic / avg_launch_s / 1e9 / 8000.0,
+                                   "mfma_tflops": achieved, "algorithmic_bytes_per_launch": traffic_algorithmic})
+    if cfg["sparse"]:
+        # the oracle multiplies a dense expansion of the block-sparse weights: its memory says nothing about the reference's
+        result["reference_saved_activation_mb"] = result["reference_peak_activation_mb"] = None
+    elif not args.no_reference_memory:
         ref_saved, ref_peak = reference_activation_memory(torch, ffn, x, dy)
         result["reference_saved_activation_mb"] = ref_saved
         result["reference_peak_activation_mb"] = ref_peak

@@ -119,11 +119,18 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
     if (kind == EPI_OUT && r == 0) return lt_launch_gemm_out(p, dtype, io_dtype, skinny_ws, skinny_bytes, stream);
     return lt_launch_gemm(p, kind, dtype, io_dtype, stream);
   }
-  LT_REQUIRE(!gated, LT_ERR_UNSUPPORTED, "internal: gated epilogue on a block-sparse projection");
   p.K[0] = lin.block;
   p.sp.mode = SPARSE_FWD; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
   p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
   p.sp.backward_indices = lin.backward_indices; p.sp.act = x; p.sp.ld_act = in; p.sp.weight = lin.weight;
+  if (gated && !(dtype == LT_BF16 && lt_sparse_mfma_supported(p, kind))) {
+    // Gate and linear output blocks have index lists of their own.  The bf16 walk for 64 x 64 blocks pairs them inside one
+    // workgroup; every other block-sparse kernel stores the pre-activation and leaves the activation to a pass of its own.
+    p.N = out;
+    p.epi = epi_store_params(epi.pre, epi.ld_pre, dtype, epi.bias);
+    LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));
+    return lt_act_forward(T, epi.inter, 1, epi.act, dtype, epi.pre, epi.hid, stream);
+  }
   return lt_launch_gemm_sparse(p, kind, dtype, io_dtype, stream);
 }
 
@@ -352,12 +359,7 @@ extern "C" int lt_ffn_forward(const lt_ffn_desc* desc, const void* x, void* y, c
                        nullptr, false, stream));
 
   // up-projection + activation
-  if (d.i2h.block > 0 && d.gated) {
-    // the block-sparse walk has no paired-column epilogue: store P, then a separate activation pass
-    EpiParams e = epi_store_params(saved->pre_activation, N1, cdt, d.i2h.bias);
-    LT_TRY(linear_forward_impl(d.i2h, T, cdt, s.u, EPI_STORE, e, saved->i2h_lowrank_hid, io, stream, s.skinny, s.skinny_bytes));
-    LT_TRY(lt_act_forward(T, I, 1, d.act, cdt, saved->pre_activation, s.hid, stream));
-  } else {
+  {
     EpiParams e;
     memset(&e, 0, sizeof(e));
     e.bias = d.i2h.bias; e.pre = saved->pre_activation; e.ld_pre = N1; e.hid = s.hid; e.ld_hid = I;

@@ -269,7 +269,8 @@ bool lt_sparse_mfma_supported(const GemmProblem& p, int kind) {
   const SparseWalk& sp = p.sp;
   const EpiParams& e = p.epi;
   if (sp.mode == SPARSE_NONE || sp.block != 64 || p.M <= 0) return false;
-  if (kind == EPI_ACT_FWD && e.gated) return false;
+  // gated forward epilogue: p.N counts the gate columns; the walk pairs gate block j with linear block j + N / 64
+  if (kind == EPI_ACT_FWD && e.gated && (sp.mode != SPARSE_FWD || p.N % 64 != 0 || e.inter != p.N)) return false;
   if (sp.ld_act % 8 != 0 || !lt_aligned(sp.act, 16)) return false;
   if (sp.mode == SPARSE_DW) {
     if (kind != EPI_STORE || sp.ld_act2 % 8 != 0 || !lt_aligned(sp.act2, 16) || !lt_aligned(e.out, 16)) return false;
@@ -296,6 +297,7 @@ int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtyp
   const SparseWalk& sp = p.sp;
   const double steps = sp.mode == SPARSE_FWD ? sp.blocks_per_out : sp.blocks_per_in;
   double flops = 2.0 * (double)p.M * (double)p.N * (steps * 64.0 + (p.nseg > 1 ? (double)p.K[1] : 0.0));
+  if (kind == EPI_ACT_FWD && p.epi.gated) flops *= 2.0;
   if (sp.mode == SPARSE_DW) flops = 2.0 * (double)sp.tokens * (double)(p.N / 64) * sp.blocks_per_in * 4096.0;
   static const char* tags[4] = {"", "blocksparse_fwd_bf16", "blocksparse_dx_bf16", "blocksparse_dw_bf16"};
   LtProfileScope scope(tags[sp.mode], flops, 0.0, stream);

@@ -95,15 +95,24 @@ template <int N, typename F> __device__ __forceinline__ void lt_static_for(F&& f
   lt_static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX, int SP = SPARSE_NONE>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
+// PH = 2 (block-sparse forward with the gated activation epilogue only): a workgroup owns gate block tn and the matching
+// linear block tn + N / 64, which have index lists of their own.  It walks the two lists one after the other (two phases
+// over the same LDS stages) into two sets of accumulators and pairs them in the epilogue, so the gated activation needs no
+// pass of its own over the pre-activations.
+template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX, int SP = SPARSE_NONE, int PH = 1>
+__global__ __launch_bounds__(WM * WN * 64)
+__attribute__((amdgpu_waves_per_eu(SP != SPARSE_NONE ? 2 : 1)))  // the block-sparse walks: two workgroups per CU (their LDS allows it)
+void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int NT = WM * WN * 64;
+  static_assert(PH == 1 || (PH == 2 && SP == SPARSE_FWD && KIND == EPI_ACT_FWD && WN == 1), "two phases: gated block-sparse forward");
   static_assert(SP == SPARSE_NONE || (SP == SPARSE_FWD && A_KM && B_KM && BN == 64) ||
                     (SP == SPARSE_DX && A_KM && !B_KM && BN == 64) ||
                     (SP == SPARSE_DW && !A_KM && !B_KM && BM == 256 && BN == 64 && WM == 4 && WN == 1),
                 "operand layouts and tile shape of the block-sparse walks");
-  constexpr int WTM = BM / WM, WTN = BN / WN;
-  constexpr int FM = WTM / 32, FN = WTN / 32;
+  constexpr int WTM = BM / WM;
+  constexpr int WTN_IN = BN / WN, FN_IN = WTN_IN / 32;  // columns / column blocks of a wavefront in one phase
+  constexpr int WTN = WTN_IN * PH, FN = FN_IN * PH;     // ... and of its output sub-tile
+  constexpr int FM = WTM / 32;
   constexpr int A_CHUNKS = BM * BK / 8 / NT, B_CHUNKS = BN * BK / 8 / NT;  // 16-byte chunks per thread per stage
   static_assert(BM * BK / 8 % NT == 0 && BN * BK / 8 % NT == 0, "tile must divide over the threads");
   static_assert(FN % 2 == 0 || KIND != EPI_ACT_FWD, "gated pairing needs an even number of column blocks per wavefront");
@@ -120,17 +129,30 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
   const int wm = wave / WN, wn = wave % WN;
   const bool gated = (KIND == EPI_ACT_FWD) && p.epi.gated;
 
+#ifdef LT_TILE_TIMING
+  // (the FWD / DX walks have no use for the weight-gradient walk's second activation pointer: the timing buffer rides there)
+  unsigned long long* const tile_stamps =
+      ((SP == SPARSE_FWD || SP == SPARSE_DX) && p.sp.act2)
+          ? reinterpret_cast<unsigned long long*>(const_cast<void*>(p.sp.act2)) + (size_t)blockIdx.x * 8 : nullptr;
+#endif
+  LT_TILE_STAMP(0);
+  LT_TILE_STAMP_REALTIME(4);
   // ---- tile assignment: XCD-contiguous, grouped along M
   int pid = blockIdx.x;
   const int num_pid = tiles_m * tiles_n;
   if ((num_pid & 7) == 0) pid = (pid & 7) * (num_pid >> 3) + (pid >> 3);
-  const int group = GROUP_M * tiles_n;
-  const int first_m = (pid / group) * GROUP_M;
-  const int gsz = min(tiles_m - first_m, GROUP_M);
+  // Block-sparse FWD / DX: the workgroups of one token tile gather column blocks of the same 256 activation rows (a few MiB
+  // that stay in the XCD's L2) while every block column has a weight list of its own, so one XCD's concurrent workgroups
+  // take one token tile and consecutive block columns.
+  constexpr int GROUP_ROWS = (SP == SPARSE_FWD || SP == SPARSE_DX) ? 1 : GROUP_M;
+  const int group = GROUP_ROWS * tiles_n;
+  const int first_m = (pid / group) * GROUP_ROWS;
+  const int gsz = min(tiles_m - first_m, GROUP_ROWS);
   const int tm = first_m + (pid % group) % gsz;
   const int tn = (pid % group) / gsz;
   const int64_t m0 = (int64_t)tm * BM;
-  const int64_t n0 = (int64_t)tn * (gated ? BN / 2 : BN);  // gated: in gate columns; sparse FWD / DX: tn = block index
+  // gated: in gate columns; sparse FWD / DX: tn = block index (two phases: the gate block)
+  const int64_t n0 = (int64_t)tn * ((gated && PH == 1) ? BN / 2 : BN);
 
   f32x16 acc[FM][FN];
 #pragma unroll
@@ -163,18 +185,18 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       dw_ob[j] = sp.backward_indices[(int64_t)dw_ib * sp.blocks_per_in + min(dw_a0 + j, sp.blocks_per_in - 1)];
   }
 
-  // global -> registers for k-step kt
-  auto load_tiles = [&](int kt) {
+  // global -> registers for k-step kt (ph: 0 = the tile's own block column, 1 = the matching linear block column)
+  auto load_tiles = [&](int kt, int ph = 0) {
     const int seg = kt >= kt_seg0;
     int64_t k0 = (int64_t)(seg ? kt - kt_seg0 : kt) * BK;
     int64_t K = p.K[seg];
     const bf16* A = reinterpret_cast<const bf16*>(p.A[seg].ptr);
     const bf16* B = reinterpret_cast<const bf16*>(p.B[seg].ptr);
     int64_t lda = p.A[seg].ld, ldb = p.B[seg].ld;
-    int64_t b_row0 = n0;  // first B row (k-major) / column (mn-major) of this tile
+    int64_t b_row0 = n0 + (PH == 2 ? ph * p.N : 0);  // first B row (k-major) / column (mn-major) of this tile
     if constexpr (SP == SPARSE_FWD) {
       if (!seg) {  // A: column block ib of X; B: weight block f, a [64 rows][64 k] matrix of its own
-        const int f = sp.forward_indices[(int64_t)tn * sp.blocks_per_out + kt];
+        const int f = sp.forward_indices[(int64_t)(tn + (PH == 2 ? ph * tiles_n : 0)) * sp.blocks_per_out + kt];
         A = reinterpret_cast<const bf16*>(sp.act); lda = sp.ld_act; k0 = (int64_t)(f / sp.blocks_per_in) * 64;
         B = reinterpret_cast<const bf16*>(sp.weight) + (int64_t)f * 4096; ldb = 64; b_row0 = 0;
         K = k0 + 64;
@@ -213,7 +235,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
       if constexpr (B_KM) {
         const int row = q >> 3, c = q & 7;
         int64_t gn;
-        if (gated) {
+        if (gated && PH == 1) {
           const int rr = row % WTN;
           gn = (rr / (WTN / 2)) * p.N + n0 + (row / WTN) * (WTN / 2) + rr % (WTN / 2);
         } else {
@@ -274,19 +296,19 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     return u.v;
   };
 
-  auto load_frags = [&](int s, int kk, bf16x8 (&a)[FM], bf16x8 (&b)[FN]) {
+  auto load_frags = [&](int s, int kk, bf16x8 (&a)[FM], bf16x8 (&b)[FN_IN]) {
 #pragma unroll
     for (int i = 0; i < FM; i++) {
       if constexpr (A_KM) a[i] = frag_km(lds_a[s], wm * WTM + i * 32, kk);
       else a[i] = frag_mn(lds_a[s], std::integral_constant<int, BM>{}, wm * WTM + i * 32, kk);
     }
 #pragma unroll
-    for (int j = 0; j < FN; j++) {
-      if constexpr (B_KM) b[j] = frag_km(lds_b[s], wn * WTN + j * 32, kk);
-      else b[j] = frag_mn(lds_b[s], std::integral_constant<int, BN>{}, wn * WTN + j * 32, kk);
+    for (int j = 0; j < FN_IN; j++) {
+      if constexpr (B_KM) b[j] = frag_km(lds_b[s], wn * WTN_IN + j * 32, kk);
+      else b[j] = frag_mn(lds_b[s], std::integral_constant<int, BN>{}, wn * WTN_IN + j * 32, kk);
     }
   };
-  constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);  // LDS read instructions per k-substep
+  constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN_IN * (B_KM ? 1 : 2);  // LDS read instructions per k-substep
 
   // split-k: this workgroup's slice of the k-steps
   int kt_begin = 0, kt_end = kt_total;
@@ -295,18 +317,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     kt_begin = min(kt_total, (int)blockIdx.y * per);
     kt_end = min(kt_total, kt_begin + per);
   }
-  if (kt_begin < kt_end) {
-    load_tiles(kt_begin);
-    store_tiles(kt_begin & 1);
-  }
-  __syncthreads();
-  for (int kt = kt_begin; kt < kt_end; kt++) {
-    const int s = kt & 1;
-    const bool has_next = kt + 1 < kt_end;
-    if (has_next) load_tiles(kt + 1);
-    // fragments are double-buffered in registers: the LDS reads of k-substep kk + 1 are issued before, and interleaved
-    // with, the MFMAs of k-substep kk
-    bf16x8 af[2][FM], bfr[2][FN];
+  // the matrix instructions of one k-step on LDS stage s.  Fragments are double-buffered in registers: the LDS reads of
+  // k-substep kk + 1 are issued before, and interleaved with, the MFMAs of k-substep kk
+  auto multiply_stage = [&](int s, auto PHASE) __attribute__((always_inline)) {
+    constexpr int j0 = decltype(PHASE)::value * FN_IN;  // this phase's accumulator columns
+    bf16x8 af[2][FM], bfr[2][FN_IN];
     load_frags(s, 0, af[0], bfr[0]);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; kk++) {
@@ -314,13 +329,29 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
 #pragma unroll
       for (int i = 0; i < FM; i++)
 #pragma unroll
-        for (int j = 0; j < FN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
-      if (kk + 1 < BK / 16) SchedInterleave<FRAG_READS, FM * FN>::run();
+        for (int j = 0; j < FN_IN; j++)
+          acc[i][j0 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j0 + j], 0, 0, 0);
+      if (kk + 1 < BK / 16) SchedInterleave<FRAG_READS, FM * FN_IN>::run();
     }
-    if (has_next) store_tiles(s ^ 1);
+  };
+  LT_TILE_STAMP(1);
+  lt_static_for<PH>([&](auto PHASE) __attribute__((always_inline)) {
+    constexpr int ph = decltype(PHASE)::value;
+    if (kt_begin < kt_end) {
+      load_tiles(kt_begin, ph);
+      store_tiles(kt_begin & 1);
+    }
     __syncthreads();
-  }
+    for (int kt = kt_begin; kt < kt_end; kt++) {
+      const int s = kt & 1;
+      const bool has_next = kt + 1 < kt_end;
+      if (has_next) load_tiles(kt + 1, ph);
+      multiply_stage(s, PHASE);
+      if (has_next) store_tiles(s ^ 1);
+      __syncthreads();
+    }
+  });
+  LT_TILE_STAMP(2);
 
   // ---- epilogue.  The accumulators of a 32 x 32 block sit column-per-lane (register r = row 8 * (r / 4) + 4 * (lane / 32)
   //      + r % 4, column lane % 32); each wavefront transposes one 32-row strip of its sub-tile at a time through its own
@@ -456,8 +487,38 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
     }
     __builtin_amdgcn_wave_barrier();
   };
+  // forward activation, tanh GELU, h stored: the gate (or only) half and the linear half of a strip are read back from the
+  // stage with all LDS loads issued before the first value is used
+  auto act_fwd_strip = [&](auto I, auto G) __attribute__((always_inline)) {
+    constexpr int i = decltype(I)::value;
+    constexpr bool GATED = decltype(G)::value;
+    constexpr int LPR = (GATED ? WTN / 2 : WTN) / 8, RPI = 64 / LPR, NITF = 32 / RPI;
+    const int c = (lane % LPR) * 8;
+    const int64_t n = n0 + wn * (GATED ? WTN / 2 : WTN) + c;
+    const int64_t mlane = m_base + wm * WTM + i * 32 + lane / LPR;
+    stage_strip(I);
+    float vg[NITF][8], vl[GATED ? NITF : 1][8];
+#pragma unroll
+    for (int it = 0; it < NITF; it++) {
+      const float* sv = &stage[(it * RPI + lane / LPR) * STAGE_LD + c];
+#pragma unroll
+      for (int e = 0; e < 8; e++) vg[it][e] = sv[e];
+      if constexpr (GATED) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) vl[it][e] = sv[WTN / 2 + e];
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NITF; it++) epi_act_fwd8_gelu<GATED>(epi, mlane + it * RPI, n, vg[it], vl[GATED ? it : 0]);
+    __builtin_amdgcn_wave_barrier();
+  };
   const bool whole_tile = m_base + BM <= m_limit;
-  if constexpr (NIT <= 4 && KIND == EPI_STORE) {
+  if constexpr (KIND == EPI_ACT_FWD && SP != SPARSE_NONE) {
+    const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED && epi.hid != nullptr && epi.pre != nullptr;
+    if (straight && pair) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { act_fwd_strip(I, std::true_type{}); });
+    else if (straight) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { act_fwd_strip(I, std::false_type{}); });
+    else lt_static_for<FM>(generic_strip);
+  } else if constexpr (NIT <= 4 && KIND == EPI_STORE) {
     if (whole_tile && epi.out_dtype == LT_F32) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { store_strip(I, float{}); });
     else if (whole_tile) lt_static_for<FM>([&](auto I) __attribute__((always_inline)) { store_strip(I, bf16{}); });
     else lt_static_for<FM>(generic_strip);
@@ -493,6 +554,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(GemmProblem p, 
   } else {
     lt_static_for<FM>(generic_strip);
   }
+  LT_TILE_STAMP(3);
+  LT_TILE_STAMP_REALTIME(5);
 }
 
 // =====================================================================================================================
@@ -1267,7 +1330,15 @@ int launch_cfg(const GemmProblem& p, int io_dtype, hipStream_t stream) {
   return LT_OK;
 }
 
-template <int KIND> int launch_sparse(const GemmProblem& p, int io_dtype, hipStream_t stream) {
+template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
+  GemmProblem p = problem;
+#ifdef LT_TILE_TIMING
+  // block-sparse FWD / DX launch number i of the process writes region i % 4 (8192 workgroups each) of its own buffer
+  if (const char* e = getenv("LT_TILE_TIMING_BUFFER_SPARSE")) {
+    if (p.sp.mode == SPARSE_FWD || p.sp.mode == SPARSE_DX)
+      p.sp.act2 = (const void*)(strtoull(e, nullptr, 0) + (size_t)(lt_tile_timing_launch_counter()++ % 4) * 8192 * 64);
+  }
+#endif
   const SparseWalk& sp = p.sp;
   const bool bf16_io = KIND == EPI_OUT && io_dtype == LT_BF16;
   dim3 block(256);
@@ -1275,7 +1346,11 @@ template <int KIND> int launch_sparse(const GemmProblem& p, int io_dtype, hipStr
     const int tiles_m = (int)((p.M + 255) / 256), groups = (int)(p.N / 64);
     dim3 grid((unsigned)(tiles_m * groups));
     using TXB = std::conditional_t<KIND == EPI_OUT, bf16, float>;  // only EPI_OUT touches x / y
-    if (sp.mode == SPARSE_FWD) {
+    if (sp.mode == SPARSE_FWD && KIND == EPI_ACT_FWD && p.epi.gated) {
+      // p.N counts the gate columns: one workgroup per (token tile, gate block), paired with linear block tn + groups
+      if constexpr (KIND == EPI_ACT_FWD)
+        hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, true, EPI_ACT_FWD, float, SPARSE_FWD, 2>), grid, block, 0, stream, p, tiles_m, groups);
+    } else if (sp.mode == SPARSE_FWD) {
       if (bf16_io) hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, true, KIND, TXB, SPARSE_FWD>), grid, block, 0, stream, p, tiles_m, groups);
       else hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, true, true, KIND, float, SPARSE_FWD>), grid, block, 0, stream, p, tiles_m, groups);
     } else {

@@ -456,6 +456,8 @@ int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_
 // algorithmic flops of a dense problem: 2 * M * N * (K0 + K1)
 double lt_gemm_flops(const GemmProblem& p, int kind);
 // block-sparse walk: matrix-core kernel for 64 x 64 bf16 blocks, else the any-shape kernel
+// whether the bf16 matrix-core walk for 64 x 64 blocks takes this block-sparse problem with epilogue `kind`
+bool lt_sparse_mfma_supported(const GemmProblem& p, int kind);
 int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);
 // EPI_STORE problems with few output tiles and a long reduction (the low-rank factors of a generalized linear layer):
 // 128 x 128 tiles, the reduction split over workgroups through `workspace` when that fills the chip better.  Falls back to

@@ -1,13 +1,16 @@
 """Where the cycles of each GEMM launch of a LeanFFN step go: prologue, main loop, epilogue, per workgroup (= per tile).
 
     python -m lean_transformer_amd._build --tile-timing      (once: builds csrc/libleanffn_tile_timing.so)
-    python -m lean_transformer_amd.tile_timing --config c3    (on the GPU)
+    python -m lean_transformer_amd.tile_timing --config c3    (on the GPU; c2: the other dense configuration; c4: the
+                                                               block-sparse one)
 
 Runs fwd+bwd steps of a benchmark configuration (bench.py's) on the instrumented library, in which thread 0 of every
 workgroup of the copy-based GEMM kernel stamps the shader clock (s_memtime) at its phase boundaries and the 100 MHz
 real-time counter at both ends.  Prints, per launch of a step: tiles, wall-clock span, shader-clock ticks per tile split
 into prologue (launch to first matrix instruction), main loop (with the first 16 k-steps apart) and epilogue, the ideal
 (1 024 ticks per 32-wide k-step: 32 matrix instructions of 32 cycles per SIMD) and the shader clock while tiles run.
+With --config c4 the stamped kernels are the block-sparse forward / input-gradient walks (256 x 64 tiles, two workgroups per
+CU): start, before the first operand loads, after the main loop, after the epilogue.
 A measurement tool: nothing in the package imports it.
 """
 import argparse
@@ -17,7 +20,7 @@ import sys
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", default="c3", choices=["c2", "c3"], help="dense bf16 benchmark configuration of bench.py")
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4"], help="bf16 benchmark configuration of bench.py")
     ap.add_argument("--warmup", type=int, default=20)
     args = ap.parse_args()
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -36,6 +39,8 @@ def main():
     cfg = bench.CONFIGS[args.config]
     ffn, x, dy = bench.build_workload(torch, lt, cfg, dev)
     params = list(ffn.parameters())
+    if cfg["sparse"]:
+        return sparse_walks(torch, ffn, x, dy, params, cfg, dev)
     regions, slots = 6, 4096
     stamps = torch.zeros(regions * slots * 8, dtype=torch.int64, device=dev)
     os.environ["LT_TILE_TIMING_BUFFER"] = hex(stamps.data_ptr())
@@ -73,6 +78,43 @@ def main():
               f"{(loop.mean() - first16) / (ksteps - 16):6.1f})  epilogue {epilogue.mean():6.0f} (max {epilogue.max():6d})  "
               f"clock {clock:.3f} GHz")
     print(f"all six launches: matrix-core-ideal ticks / measured ticks = {total_ideal / total_ticks:.3f}")
+
+
+def sparse_walks(torch, ffn, x, dy, params, cfg, dev):
+    """the four block-sparse FWD / DX launches of a step: launch i of the process writes region i % 4 (8192 workgroups each)"""
+    regions, slots = 4, 8192
+    stamps = torch.zeros(regions * slots * 8, dtype=torch.int64, device=dev)
+    os.environ["LT_TILE_TIMING_BUFFER_SPARSE"] = hex(stamps.data_ptr())
+
+    def step():
+        y = ffn(x)
+        torch.autograd.grad(y, [x, *params], dy)
+
+    for _ in range(20):
+        step()
+    torch.cuda.synchronize()
+    stamps.zero_()
+    step()
+    torch.cuda.synchronize()
+    data = stamps.cpu().numpy().reshape(regions, slots, 8)
+    hidden, inter = cfg["hidden"], cfg["inter"]
+    n1 = 2 * inter if cfg["gated"] else inter
+    per_out_up, per_out_down = ffn.i2h_proj.matrix.forward_indices.shape[1], ffn.h2o_proj.matrix.forward_indices.shape[1]
+    per_in_up, per_in_down = ffn.i2h_proj.matrix.backward_indices.shape[1], ffn.h2o_proj.matrix.backward_indices.shape[1]
+    rank_steps = ffn.i2h_proj.matrix.lowrank_first.shape[0] // 64 if ffn.i2h_proj.matrix.lowrank_first is not None else 0
+    gated = 2 if cfg["gated"] else 1  # the gated up-projection walks the gate block's and the linear block's list
+    launches = [("up-projection + activation", gated * (per_out_up + rank_steps)), ("down-projection + residual", per_out_down + rank_steps),
+                ("dh + d-activation", per_in_down + rank_steps), ("du", per_in_up + rank_steps)]
+    print(f"{cfg['name']}\nticks = shader clock cycles per 256 x 64 tile (two workgroups share a CU); k-step = one 64 x 64 weight block; "
+          "a workgroup's matrix instructions of a k-step take 512 ticks of its SIMDs")
+    for (label, ksteps), d in zip(launches, data):
+        d = d[d[:, 3] != 0]
+        prologue, loop, epilogue = d[:, 1] - d[:, 0], d[:, 2] - d[:, 1], d[:, 3] - d[:, 2]
+        clock = ((d[:, 3] - d[:, 0]) / ((d[:, 5] - d[:, 4]) * 10.0)).mean()
+        span = (d[:, 5].max() - d[:, 4].min()) / 100.0
+        print(f"{label:28s} tiles {len(d):5d}  span {span:7.1f} us  ticks/tile {(d[:, 3] - d[:, 0]).mean():9.0f}  before the loop "
+              f"{prologue.mean():6.0f}  loop {loop.mean():9.0f} = {loop.mean() / ksteps:6.1f}/k-step ({ksteps} k-steps)  "
+              f"epilogue {epilogue.mean():6.0f}  clock {clock:.3f} GHz")
 
 
 if __name__ == "__main__":

@@ -90,7 +90,7 @@ class LinearParams:
         for ib in range(n_in):
             for a in range(A):
                 blocks[bwd[ib][a]][ib] = w4[ib, a]
-        zero = torch.zeros(b, b, dtype=self.weight.dtype)
+        zero = torch.zeros(b, b, dtype=self.weight.dtype, device=self.weight.device)
         for ob in range(n_out):
             rows.append(torch.cat([blk if blk is not None else zero for blk in blocks[ob]], dim=1))
         return torch.cat(rows, dim=0)
