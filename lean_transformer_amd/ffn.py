@@ -203,7 +203,9 @@ class _LeanFFN(torch.autograd.Function):
             ctx, tokens, hidden, ln_weight, ln_bias, i2h_weight, i2h_bias, i2h_lowrank_first, i2h_lowrank_second,
             i2h_forward_indices, i2h_backward_indices, h2o_weight, h2o_bias, h2o_lowrank_first, h2o_lowrank_second,
             h2o_forward_indices, h2o_backward_indices, post_ln_weight, post_ln_bias, io)
-        # fp32 copies of the small vectors (LayerNorm parameters, biases): backward reuses them instead of converting again
+        # fp32 copies of the small vectors (LayerNorm parameters, biases): backward reuses them instead of converting again.
+        # The parameters themselves go through save_for_backward below, so an in-place update between forward and backward
+        # makes ctx.saved_tensors raise (autograd's version check) before these copies could be used stale.
         ctx._small_fp32 = (keep[0], keep[1], keep[2], keep[3], keep[4][1], keep[5][1])
         n1 = desc.i2h.out_features
         y = torch.empty_like(x)

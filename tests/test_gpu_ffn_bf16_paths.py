@@ -219,3 +219,15 @@ def test_bf16_dense_generalized_linear_alone(tokens, lowrank_dim, adapter_dim, b
     assert_close(grads[0], ref[0], BF16, "dx")
     for name, a, b in zip(names, grads[1:], ref[1:]):
         assert_close(a, b, BF16, name)
+
+
+def test_in_place_parameter_update_between_forward_and_backward_is_refused():
+    """backward reuses fp32 copies of the LayerNorm parameters and biases made in forward; the parameters themselves are
+    saved for backward, so updating one in place before backward raises instead of pairing stale copies with fresh weights"""
+    ffn = lt.LeanFFN(256, 512, gated=True).to(DEV).to(BF16)
+    x = torch.randn(64, 256, device=DEV, dtype=BF16, requires_grad=True)
+    y = ffn(x)
+    with torch.no_grad():
+        ffn.pre_layer_norm.weight.mul_(2.0)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        y.sum().backward()
