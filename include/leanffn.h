@@ -56,6 +56,10 @@ typedef struct lt_linear {
   int32_t block;          /* sparse block size, 0 when dense */
   int32_t blocks_per_out; /* K: active blocks per output block row */
   int32_t blocks_per_in;  /* A: active blocks per input block column */
+  int32_t out_group;      /* sparse: every aligned run of this many consecutive output blocks has the same list of input
+                             blocks (PixelFly with stretch=True on a tall matrix: out_blocks / in_blocks).  A promise by the
+                             caller that only selects a faster weight-gradient kernel; 0 or 1 when not known. */
+  int32_t reserved;       /* 0 */
 } lt_linear;
 
 /* Where lt_linear_backward / lt_ffn_backward write parameter gradients; a NULL member skips that gradient.

@@ -34,7 +34,7 @@ class LtLinear(ctypes.Structure):
         ("weight", c_void_p), ("bias", c_void_p), ("lowrank_first", c_void_p), ("lowrank_second", c_void_p),
         ("forward_indices", c_void_p), ("backward_indices", c_void_p),
         ("in_features", c_int32), ("out_features", c_int32), ("lowrank", c_int32), ("block", c_int32),
-        ("blocks_per_out", c_int32), ("blocks_per_in", c_int32),
+        ("blocks_per_out", c_int32), ("blocks_per_in", c_int32), ("out_group", c_int32), ("reserved", c_int32),
     ]
 
 

@@ -139,6 +139,26 @@ def _as(t: Optional[torch.Tensor], dtype: torch.dtype) -> Optional[torch.Tensor]
     return t.contiguous()
 
 
+def shared_list_run(forward_indices: torch.Tensor, blocks_per_in: int) -> int:
+    """Largest power of two g such that every aligned run of g consecutive output blocks has the same list of input blocks
+    (1 when neighbouring output blocks differ).  PixelFly with ``stretch=True`` on a matrix with more output than input
+    blocks repeats every list ``out_blocks / in_blocks`` times; the weight-gradient kernel reads dY once per run of 4
+    instead of once per output block when told so.  Computed once per index tensor (one device -> host sync) and remembered
+    on the tensor object itself together with the tensor's version counter, so an in-place change recomputes it."""
+    cached = getattr(forward_indices, "_lt_shared_list_run", None)
+    if cached is not None and cached[0] == (forward_indices._version, blocks_per_in):
+        return cached[1]
+    lists = torch.div(forward_indices, blocks_per_in, rounding_mode="floor")  # input block of every entry
+    run, n_out = 1, lists.shape[0]
+    while n_out % (2 * run) == 0:
+        grouped = lists.reshape(n_out // (2 * run), 2 * run, -1)
+        if not bool((grouped == grouped[:, :1]).all()):
+            break
+        run *= 2
+    forward_indices._lt_shared_list_run = ((forward_indices._version, blocks_per_in), run)
+    return run
+
+
 def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices, backward_indices) -> "nat.LtLinear":
     """ctypes descriptor of one projection; all tensors already in their final dtype and contiguous"""
     desc = nat.LtLinear()
@@ -154,6 +174,7 @@ def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices
         desc.in_features, desc.out_features = in_features, forward_indices.shape[0] * block
         desc.block, desc.blocks_per_in, desc.blocks_per_out = block, blocks_per_in, forward_indices.shape[1]
         desc.forward_indices, desc.backward_indices = nat.ptr(forward_indices), nat.ptr(backward_indices)
+        desc.out_group = shared_list_run(forward_indices, blocks_per_in) if forward_indices is not None else 0
     return desc
 
 

@@ -218,6 +218,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.act2 = x_act;
       p.sp.ld_act2 = in; p.sp.tokens = T;
+      p.sp.out_group = lin.forward_indices ? lin.out_group : 0;  // the grouped kernel reads the list from the forward table
       p.epi = epi_store_params(grads.weight, lin.block, dtype, nullptr);
       LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));
     }

@@ -652,6 +652,25 @@ template <bool KM> struct DmaOperand {
     unit_bytes = KM ? 64 * 2 : DK * ld * 2;
   }
 
+  // mn-major operand whose 256 tile columns are four 64-wide column blocks gathered from anywhere in the matrix: block j of
+  // the tile is the operand's column block blocks[j]
+  __device__ __forceinline__ void setup_gather(const GemmOperand& op, const int (&blocks)[4], int wave, int lane) {
+    static_assert(!KM, "column blocks are gathered for mn-major operands");
+    seg = 0;
+    const int64_t ld = op.ld;
+#pragma unroll
+    for (int j = 0; j < LOADS; j++) {
+      const int q = (wave * LOADS + j) * 64 + lane;
+      const int kr = q >> 5, c = (q & 31) ^ swz_mn(kr);
+      const int slot = c >> 3;
+      const int blk = slot == 0 ? blocks[0] : slot == 1 ? blocks[1] : slot == 2 ? blocks[2] : blocks[3];
+      off[j] = (uint32_t)((kr * ld + (int64_t)blk * 64 + (c & 7) * 8) * 2);
+      krow[j] = kr;
+    }
+    base = reinterpret_cast<const char*>(op.ptr);
+    unit_bytes = DK * ld * 2;
+  }
+
   // all copies of unit u (counted inside the k-segment) into `dst`; k_limit: reduction length for the ragged test
   // J0, J1: range of this wavefront's copy instructions (a k-major block can go out in two halves)
   template <bool K_TAIL, int J0 = 0, int J1 = LOADS>
@@ -731,7 +750,10 @@ constexpr bool SPLIT_MN_B = true;
 // m0 + wm * WTM + 32 i, columns n0 + wn * 128 + 32 j of the result (gated forward: blocks 0, 1 gate columns, 2, 3 the
 // matching linear columns).  `stage` is 16 KiB of LDS that belongs to this wavefront alone; tile_rows x tile_cols is the
 // workgroup's tile (for the whole-tile test).  The bias is already in the accumulators.
-template <int FM, int KIND, typename TX, int tile_rows, int tile_cols>
+// SCATTER (EPI_STORE only; the grouped block-sparse weight gradient): the tile is 4 output blocks (rows) x 4 entries of
+// their shared list of input blocks (columns); each 64 x 64 piece goes to its own block of the native [in, A, block] weight
+// gradient, at the flat position the forward table names.  List entries past the end (the last column tile) are not stored.
+template <int FM, int KIND, typename TX, int tile_rows, int tile_cols, bool SCATTER = false>
 __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const GemmProblem& p, float* stage, const int64_t m0,
                                                   const int64_t n0, const int wm, const int wn, const bool gated) {
   constexpr int FN = 4, WTN = 128, WTM = FM * 32;
@@ -905,7 +927,30 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
     }
     __builtin_amdgcn_wave_barrier();
   };
-  if constexpr (KIND == EPI_ACT_BWD) {
+  auto scatter_strip = [&](auto I, auto out_type) {
+    using TO = decltype(out_type);
+    constexpr int i = decltype(I)::value;
+    constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
+    const int c = (lane % LANES_PER_ROW) * 8;
+    const int per_out = p.sp.blocks_per_out;
+    const int64_t ob = m0 / 64 + (wm * WTM + i * 32) / 64;
+    const int entry = (int)(n0 / 64) + wn * 2 + (c >> 6);  // position in the output block's list
+    const int64_t flat = p.sp.forward_indices[ob * per_out + min(entry, per_out - 1)];
+    TO* dst = reinterpret_cast<TO*>(epi.out) + flat * 4096 + ((i & 1) * 32 + lane / LANES_PER_ROW) * 64 + (c & 63);
+    stage_strip(I);
+    float v[NIT][8];
+    read_staged_rows(std::integral_constant<int, NIT>{}, std::integral_constant<int, ROWS_PER_IT>{}, LANES_PER_ROW, c, v);
+    if (entry < per_out) {
+#pragma unroll
+      for (int it = 0; it < NIT; it++) store8(dst + it * ROWS_PER_IT * 64, v[it]);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  if constexpr (SCATTER) {
+    static_assert(KIND == EPI_STORE, "scattered blocks: plain store");
+    if (epi.out_dtype == LT_F32) for_each_strip([&](auto I) { scatter_strip(I, float{}); });
+    else for_each_strip([&](auto I) { scatter_strip(I, bf16{}); });
+  } else if constexpr (KIND == EPI_ACT_BWD) {
     const bool straight = whole_tile && epi.act == LT_ACT_GELU_FUSED && epi.hid != nullptr;
     if (straight && epi.gated) for_each_strip([&](auto I) { act_bwd_strip(I, std::true_type{}); });
     else if (straight) for_each_strip([&](auto I) { act_bwd_strip(I, std::false_type{}); });
@@ -952,8 +997,12 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
   }
 }
 
-template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL>
+// GATHER (both operands mn-major, plain store): the grouped block-sparse weight gradient.  A = dY [tokens, out], a tile row
+// = 4 consecutive output blocks that share one list of input blocks; B = X [tokens, in], a tile column = 4 entries of that
+// list, gathered as four 64-wide column blocks; the result is scattered to the weight gradient's blocks (SCATTER above).
+template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL, bool GATHER = false>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
+  static_assert(!GATHER || (!A_KM && !B_KM && KIND == EPI_STORE && !K_TAIL), "gathered columns: weight-gradient layout");
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
   constexpr int HALF = 4;  // copy instructions per wavefront for a mn-major k-step or half a k-major block
   constexpr int KM_ELEMS = 256 * 64, MN_ELEMS = DK * 256;
@@ -1059,7 +1108,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   DmaOperand<A_KM> ca;
   DmaOperand<B_KM> cb;
   auto setup_a = [&](int seg) { ca.setup(p.A[seg], seg, m0, p.M, 0, wave, lane); };
-  auto setup_b = [&](int seg) { cb.setup(p.B[seg], seg, n0, p.N, (B_KM && gated) ? p.N : 0, wave, lane); };
+  auto setup_b = [&](int seg) {
+    if constexpr (GATHER) {
+      // the input blocks of list entries tn * 4 .. tn * 4 + 3 of output block tm * 4 (past the end: the last entry again)
+      int blocks[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int entry = min(tn * 4 + j, p.sp.blocks_per_out - 1);
+        blocks[j] = p.sp.forward_indices[(int64_t)tm * 4 * p.sp.blocks_per_out + entry] / p.sp.blocks_per_in;
+      }
+      cb.setup_gather(p.B[0], blocks, wave, lane);
+    } else {
+      cb.setup(p.B[seg], seg, n0, p.N, (B_KM && gated) ? p.N : 0, wave, lane);
+    }
+  };
   setup_a(0);
   setup_b(0);
   // copies of the unit that holds k-step t (a block for k-major operands) into the buffer of position I
@@ -1268,7 +1330,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 
   // 16 KiB of staging space per wavefront: the first two buffers of each operand
   bf16* const stage_buf = wave == 0 ? (A_KM ? a_d0 : a_s0) : wave == 1 ? (A_KM ? a_d1 : a_s1) : wave == 2 ? (B_KM ? b_d0 : b_s0) : (B_KM ? b_d1 : b_s1);
-  dma_tile_epilogue<FM, KIND, TX, BM, BN>(acc, p, reinterpret_cast<float*>(stage_buf), m0, n0, wm, wn, gated);
+  dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER>(acc, p, reinterpret_cast<float*>(stage_buf), m0, n0, wm, wn, gated);
   LT_TILE_STAMP(3);
   LT_TILE_STAMP_REALTIME(5);
   static_assert(32 * WTN * 4 <= MN_ELEMS * 2, "a 32-row strip must fit the smallest buffer");
@@ -1359,6 +1421,24 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
     }
   } else {
     if constexpr (KIND == EPI_STORE) {
+      const int64_t out_features = sp.ld_act;
+      if (sp.out_group >= 4 && sp.out_group % 4 == 0 && sp.forward_indices && out_features % 256 == 0 && sp.tokens % DK == 0 &&
+          sp.tokens > 0 && 32 * sp.ld_act * 2 + out_features * 2 < (int64_t)1 << 32 && 32 * sp.ld_act2 * 2 + p.N * 2 < (int64_t)1 << 32) {
+        // grouped: a dense both-operands-mn-major product dY^T X per run of 4 output blocks, over their shared list
+        GemmProblem q = p;
+        q.M = out_features;
+        const int tiles_m = (int)(out_features / 256), tiles_n = (sp.blocks_per_out + 3) / 4;
+        q.N = (int64_t)tiles_n * 256;
+        q.nseg = 1; q.K[0] = sp.tokens; q.K[1] = 0;
+        q.A[0].ptr = sp.act; q.A[0].ld = sp.ld_act; q.A[0].kmajor = 0;
+        q.B[0].ptr = sp.act2; q.B[0].ld = sp.ld_act2; q.B[0].kmajor = 0;
+        q.sp.act2 = nullptr;
+        q.ksplit = 0; q.krot = 0;
+        hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, true>), dim3((unsigned)(tiles_m * tiles_n)),
+                           block, 0, stream, q, tiles_m, tiles_n);
+        LT_LAUNCH_CHECK();
+        return LT_OK;
+      }
       const int groups = (int)((p.N / 64) * ((sp.blocks_per_in + 3) / 4));  // p.N = in_features
       hipLaunchKernelGGL((gemm_bf16_kernel<256, 64, 4, 1, false, false, EPI_STORE, float, SPARSE_DW>), dim3((unsigned)groups),
                          block, 0, stream, p, 1, groups);

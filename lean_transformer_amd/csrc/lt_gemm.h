@@ -63,6 +63,10 @@ struct SparseWalk {
   const void* act2;    // DW: X [tokens, in]
   int64_t ld_act2;
   int64_t tokens;      // DW: reduction length
+  // DW: every aligned run of this many consecutive output blocks shares one list of input blocks (0 / 1: not known to).
+  // With runs of 4 or more the weight gradient is computed on 256 x 256 tiles (4 output blocks x 4 input blocks of the
+  // shared list), which read every dY column block once per 4 input blocks instead of once per input block.
+  int out_group;
 };
 
 struct GemmProblem {
