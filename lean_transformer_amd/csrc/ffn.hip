@@ -123,9 +123,18 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
   p.sp.mode = SPARSE_FWD; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
   p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
   p.sp.backward_indices = lin.backward_indices; p.sp.act = x; p.sp.ld_act = in; p.sp.weight = lin.weight;
-  if (gated && !(dtype == LT_BF16 && lt_sparse_mfma_supported(p, kind))) {
-    // Gate and linear output blocks have index lists of their own.  The bf16 walk for 64 x 64 blocks pairs them inside one
-    // workgroup; every other block-sparse kernel stores the pre-activation and leaves the activation to a pass of its own.
+  p.sp.out_group = lin.out_group;
+  bool two_passes = gated && !(dtype == LT_BF16 && lt_sparse_mfma_supported(p, kind));
+  if (gated && !two_passes) {
+    // Gate and linear output blocks have index lists of their own; the bf16 walk for 64 x 64 blocks pairs them inside one
+    // workgroup.  Where the layout lets the product run on 256 x 256 tiles instead (runs of output blocks with a shared
+    // list), that and a separate activation pass are faster than the paired walk.
+    GemmProblem s = p;
+    s.N = out;
+    s.epi = epi_store_params(epi.pre, epi.ld_pre, dtype, epi.bias);
+    two_passes = lt_sparse_forward_grouped(s, EPI_STORE);
+  }
+  if (two_passes) {  // store the pre-activation, then the activation as a pass of its own
     p.N = out;
     p.epi = epi_store_params(epi.pre, epi.ld_pre, dtype, epi.bias);
     LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));

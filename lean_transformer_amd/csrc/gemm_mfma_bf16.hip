@@ -292,6 +292,20 @@ bool lt_sparse_mfma_supported(const GemmProblem& p, int kind) {
   return true;
 }
 
+bool lt_sparse_forward_grouped(const GemmProblem& p, int kind) {
+  const SparseWalk& sp = p.sp;
+  if (sp.mode != SPARSE_FWD || (kind != EPI_STORE && kind != EPI_ACT_FWD) || (kind == EPI_ACT_FWD && p.epi.gated)) return false;
+  if (!lt_sparse_mfma_supported(p, kind)) return false;
+  if (sp.out_group < 4 || sp.out_group % 4 != 0 || p.N % 256 != 0) return false;
+  // the list travels in one register: at most 64 entries, input block and flat position in 16 bits each
+  if (sp.blocks_per_out > 64 || sp.ld_act / 64 * sp.blocks_per_in > 65535) return false;
+  if (p.nseg > 1 && p.K[1] % 64 != 0) return false;
+  // 32-bit byte offsets inside a tile
+  if (256 * sp.ld_act * 2 >= (int64_t)1 << 32) return false;
+  if (p.nseg > 1 && (256 * p.A[1].ld * 2 >= (int64_t)1 << 32 || 256 * p.B[1].ld * 2 >= (int64_t)1 << 32)) return false;
+  return true;
+}
+
 int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream) {
   if (dtype != LT_BF16 || !lt_sparse_mfma_supported(p, kind)) return lt_launch_gemm_generic(p, kind, dtype, io_dtype, stream);
   const SparseWalk& sp = p.sp;

@@ -997,12 +997,21 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
   }
 }
 
-// GATHER (both operands mn-major, plain store): the grouped block-sparse weight gradient.  A = dY [tokens, out], a tile row
-// = 4 consecutive output blocks that share one list of input blocks; B = X [tokens, in], a tile column = 4 entries of that
-// list, gathered as four 64-wide column blocks; the result is scattered to the weight gradient's blocks (SCATTER above).
-template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL, bool GATHER = false>
+// Block-sparse layouts in which every aligned run of 4 consecutive output blocks shares one list of input blocks are dense
+// products over gathered operands:
+// GATHER == 1 (both operands mn-major, plain store): the weight gradient.  A = dY [tokens, out], a tile row = a run of 4
+//   output blocks; B = X [tokens, in], a tile column = 4 entries of the run's list, gathered as four 64-wide column blocks;
+//   the result is scattered to the weight gradient's blocks (SCATTER above).
+// GATHER == 2 (both operands k-major): the forward product.  A tile column = a run of 4 output blocks; k-block e of the first
+//   k-segment is entry e of the run's list: A = column block ib_e of X, B = the four weight blocks (ib_e, a_e .. a_e + 3),
+//   which are adjacent in the native [in, A, block] layout (the run's blocks are consecutive among the active output blocks of
+//   ib_e) and so form one [256 rows][64 k] k-major matrix.  The list sits in one register (lane e: ib_e << 16 | flat
+//   position) and is read with v_readlane, so the k-loop issues no memory instruction for it.  A second k-segment (the
+//   low-rank term) is an ordinary one.
+template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL, int GATHER = 0>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
-  static_assert(!GATHER || (!A_KM && !B_KM && KIND == EPI_STORE && !K_TAIL), "gathered columns: weight-gradient layout");
+  static_assert(GATHER != 1 || (!A_KM && !B_KM && KIND == EPI_STORE && !K_TAIL), "gathered columns: weight-gradient layout");
+  static_assert(GATHER != 2 || (A_KM && B_KM && !K_TAIL), "gathered k-blocks: forward layout");
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
   constexpr int HALF = 4;  // copy instructions per wavefront for a mn-major k-step or half a k-major block
   constexpr int KM_ELEMS = 256 * 64, MN_ELEMS = DK * 256;
@@ -1095,7 +1104,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   // differs between XCDs.  Measured on the up- and down-projection shapes: +16 % and +25 % for two k-major operands,
   // nothing to gain for mn-major ones.
   int rot = 0;
-  if (!K_TAIL && p.nseg == 1 && (kt_all & 1) == 0 && p.krot) {
+  if (!K_TAIL && GATHER == 0 && p.nseg == 1 && (kt_all & 1) == 0 && p.krot) {
     const unsigned bx = blockIdx.x;
     const unsigned r = (bx & 7) * (kt_all >> 3) +
                        (p.krot == 1 ? ((bx >> 3) & 3) * (kt_all >> 5) : ((bx >> 3) & 7) * (kt_all >> 6));
@@ -1107,9 +1116,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   };
   DmaOperand<A_KM> ca;
   DmaOperand<B_KM> cb;
-  auto setup_a = [&](int seg) { ca.setup(p.A[seg], seg, m0, p.M, 0, wave, lane); };
+  int list_entry = 0;  // GATHER == 2: lane e holds entry e of this tile's list
+  if constexpr (GATHER == 2) {
+    const int e = min(lane, p.sp.blocks_per_out - 1);
+    const int flat = p.sp.forward_indices[(n0 / 64) * p.sp.blocks_per_out + e];
+    list_entry = (flat / p.sp.blocks_per_in) << 16 | flat;
+  }
+  auto setup_a = [&](int seg) {
+    if (GATHER == 2 && seg == 0) {
+      const GemmOperand x = {p.sp.act, p.sp.ld_act, 1};
+      ca.setup(x, 0, m0, p.M, 0, wave, lane);  // unit u = column block u of X
+    } else {
+      ca.setup(p.A[seg], seg, m0, p.M, 0, wave, lane);
+    }
+  };
   auto setup_b = [&](int seg) {
-    if constexpr (GATHER) {
+    if (GATHER == 2 && seg == 0) {
+      const GemmOperand w = {p.sp.weight, 64, 1};
+      cb.setup(w, 0, 0, 256, 0, wave, lane);
+      cb.unit_bytes = 64 * 64 * 2;  // unit u = weight block at flat position u (and the three after it)
+      return;
+    }
+    if constexpr (GATHER == 1) {
       // the input blocks of list entries tn * 4 .. tn * 4 + 3 of output block tm * 4 (past the end: the last entry again)
       int blocks[4];
 #pragma unroll
@@ -1132,7 +1160,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       if (seg != ca.seg) setup_a(seg);
     }
     const int ks = rotated(seg ? t - kt_seg0 : t + kt_begin);
-    ca.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(A_KM ? ks >> 1 : ks, a_buf(I), wave, p.K[seg]);
+    int unit = A_KM ? ks >> 1 : ks;
+    if (GATHER == 2 && seg == 0) unit = __builtin_amdgcn_readlane(list_entry, ks >> 1) >> 16;
+    ca.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(unit, a_buf(I), wave, p.K[seg]);
   };
   auto copy_b = [&](auto steady, auto I, int t, auto J0, auto J1) {
     int seg = cb.seg;
@@ -1141,7 +1171,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
       if (seg != cb.seg) setup_b(seg);
     }
     const int ks = rotated(seg ? t - kt_seg0 : t + kt_begin);
-    cb.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(B_KM ? ks >> 1 : ks, b_buf(I), wave, p.K[seg]);
+    int unit = B_KM ? ks >> 1 : ks;
+    if (GATHER == 2 && seg == 0) unit = __builtin_amdgcn_readlane(list_entry, ks >> 1) & 0xffff;
+    cb.template issue<K_TAIL, decltype(J0)::value, decltype(J1)::value>(unit, b_buf(I), wave, p.K[seg]);
   };
 
   // ---- MFMA operand fragments: 8 k values of row / column lane % 32 of a 32-wide block
@@ -1330,7 +1362,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 
   // 16 KiB of staging space per wavefront: the first two buffers of each operand
   bf16* const stage_buf = wave == 0 ? (A_KM ? a_d0 : a_s0) : wave == 1 ? (A_KM ? a_d1 : a_s1) : wave == 2 ? (B_KM ? b_d0 : b_s0) : (B_KM ? b_d1 : b_s1);
-  dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER>(acc, p, reinterpret_cast<float*>(stage_buf), m0, n0, wm, wn, gated);
+  dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER == 1>(acc, p, reinterpret_cast<float*>(stage_buf), m0, n0, wm, wn, gated);
   LT_TILE_STAMP(3);
   LT_TILE_STAMP_REALTIME(5);
   static_assert(32 * WTN * 4 <= MN_ELEMS * 2, "a 32-row strip must fit the smallest buffer");
@@ -1408,6 +1440,20 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
     const int tiles_m = (int)((p.M + 255) / 256), groups = (int)(p.N / 64);
     dim3 grid((unsigned)(tiles_m * groups));
     using TXB = std::conditional_t<KIND == EPI_OUT, bf16, float>;  // only EPI_OUT touches x / y
+    if constexpr (KIND == EPI_STORE || KIND == EPI_ACT_FWD) {
+      if (lt_sparse_forward_grouped(p, KIND)) {
+        // runs of 4 output blocks share one list: a dense product over gathered k-blocks on 256 x 256 tiles
+        GemmProblem q = p;
+        q.K[0] = (int64_t)sp.blocks_per_out * 64;
+        q.sp.act2 = nullptr;
+        q.ksplit = 0; q.krot = 0;
+        const int tiles_n = (int)(p.N / 256);
+        hipLaunchKernelGGL((gemm_bf16_dma_kernel<true, true, KIND, float, false, 2>), dim3((unsigned)(tiles_m * tiles_n)), block, 0,
+                           stream, q, tiles_m, tiles_n);
+        LT_LAUNCH_CHECK();
+        return LT_OK;
+      }
+    }
     if (sp.mode == SPARSE_FWD && KIND == EPI_ACT_FWD && p.epi.gated) {
       // p.N counts the gate columns: one workgroup per (token tile, gate block), paired with linear block tn + groups
       if constexpr (KIND == EPI_ACT_FWD)
@@ -1434,7 +1480,7 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
         q.B[0].ptr = sp.act2; q.B[0].ld = sp.ld_act2; q.B[0].kmajor = 0;
         q.sp.act2 = nullptr;
         q.ksplit = 0; q.krot = 0;
-        hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, true>), dim3((unsigned)(tiles_m * tiles_n)),
+        hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, 1>), dim3((unsigned)(tiles_m * tiles_n)),
                            block, 0, stream, q, tiles_m, tiles_n);
         LT_LAUNCH_CHECK();
         return LT_OK;

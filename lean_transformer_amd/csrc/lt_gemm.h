@@ -63,7 +63,7 @@ struct SparseWalk {
   const void* act2;    // DW: X [tokens, in]
   int64_t ld_act2;
   int64_t tokens;      // DW: reduction length
-  // DW: every aligned run of this many consecutive output blocks shares one list of input blocks (0 / 1: not known to).
+  // FWD / DW: every aligned run of this many consecutive output blocks shares one list of input blocks (0 / 1: not known to).
   // With runs of 4 or more the weight gradient is computed on 256 x 256 tiles (4 output blocks x 4 input blocks of the
   // shared list), which read every dY column block once per 4 input blocks instead of once per input block.
   int out_group;
@@ -460,6 +460,9 @@ int lt_launch_gemm_mfma(const GemmProblem& p, int kind, int io_dtype, hipStream_
 // algorithmic flops of a dense problem: 2 * M * N * (K0 + K1)
 double lt_gemm_flops(const GemmProblem& p, int kind);
 // block-sparse walk: matrix-core kernel for 64 x 64 bf16 blocks, else the any-shape kernel
+// whether a block-sparse forward problem (plain store or non-gated activation epilogue) runs as a dense product over
+// gathered k-blocks: its output blocks come in aligned runs of 4 or more that share one list of input blocks (sp.out_group)
+bool lt_sparse_forward_grouped(const GemmProblem& p, int kind);
 // whether the bf16 matrix-core walk for 64 x 64 blocks takes this block-sparse problem with epilogue `kind`
 bool lt_sparse_mfma_supported(const GemmProblem& p, int kind);
 int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);

@@ -107,6 +107,15 @@ def sparse_walks(torch, ffn, x, dy, params, cfg, dev):
                 ("dh + d-activation", per_in_down + rank_steps), ("du", per_in_up + rank_steps)]
     print(f"{cfg['name']}\nticks = shader clock cycles per 256 x 64 tile (two workgroups share a CU); k-step = one 64 x 64 weight block; "
           "a workgroup's matrix instructions of a k-step take 512 ticks of its SIMDs")
+    # Launch i of the process writes region i % 4.  A projection whose layout lets it run as a dense product over gathered
+    # blocks (runs of output blocks with one list) is not a walk and leaves no stamps: with three stamped launches per step one
+    # region stays empty and the filled ones follow it cyclically, in launch order.
+    filled = [bool((r[:, 3] != 0).any()) for r in data]
+    if not all(filled):
+        first = (filled.index(False) + 1) % regions
+        data = [data[(first + i) % regions] for i in range(sum(filled))]
+        launches = launches[len(launches) - len(data):]
+        print(f"({regions - len(data)} launch of the step is not a block-sparse walk)")
     for (label, ksteps), d in zip(launches, data):
         d = d[d[:, 3] != 0]
         prologue, loop, epilogue = d[:, 1] - d[:, 0], d[:, 2] - d[:, 1], d[:, 3] - d[:, 2]
