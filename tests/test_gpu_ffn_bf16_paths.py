@@ -231,3 +231,73 @@ def test_in_place_parameter_update_between_forward_and_backward_is_refused():
         ffn.pre_layer_norm.weight.mul_(2.0)
     with pytest.raises(RuntimeError, match="modified by an inplace operation"):
         y.sum().backward()
+
+
+def _dense_from_native(weight, backward_indices, out_features):
+    """[out, in] dense matrix of a native block-sparse weight [in, A, block] (differentiable scatter of its blocks)"""
+    in_features, per_in, block = weight.shape
+    n_in, n_out = in_features // block, out_features // block
+    blocks = weight.reshape(n_in, per_in, block, block)
+    grid = torch.zeros(n_out, n_in, block, block, dtype=weight.dtype, device=weight.device)
+    ib = torch.arange(n_in, device=weight.device)[:, None].expand(n_in, per_in)
+    grid = grid.index_put((backward_indices.to(weight.device), ib), blocks)
+    return grid.permute(0, 2, 1, 3).reshape(out_features, in_features)
+
+
+@pytest.mark.parametrize("tokens", [256, 300, 1024])
+@pytest.mark.parametrize("fan_in,fan_out,stretch,run", [(1024, 4096, True, 4), (512, 4096, True, 8), (1024, 4096, False, 1)])
+@pytest.mark.parametrize("lowrank_dim", [0, 64])
+def test_bf16_blocksparse_layers_with_and_without_shared_list_runs(tokens, fan_in, fan_out, stretch, run, lowrank_dim):
+    """a PixelFly layer alone in bf16: stretched over a tall matrix its output blocks come in runs with one list of input
+    blocks and the forward product and the weight gradient run as dense products over gathered blocks (whole and partial token
+    tiles; token counts that are not a multiple of 32 send the weight gradient back to the walk); tiled, every output block
+    has its own list and everything is a walk.  Against fp32 stock ops on the dense expansion of the same weights."""
+    from lean_transformer_amd.blocksparse.linear import shared_list_run
+    torch.manual_seed(tokens + fan_in + lowrank_dim)
+    layout = f"pixelfly(block_size=64, stretch={stretch})"
+    layer = lt.GeneralizedLinear(lt.GeneralizedMatrix(fan_in, fan_out, layout, lowrank_dim), bias=True)
+    with torch.no_grad():
+        layer.bias.normal_(std=0.1)
+        layer.weight.normal_(std=0.05)
+        if lowrank_dim:
+            layer.matrix.lowrank_first.normal_(std=0.05)
+            layer.matrix.lowrank_second.normal_(std=0.05)
+    layer = layer.to(DEV).to(BF16)
+    matrix = layer.matrix
+    assert shared_list_run(matrix.forward_indices, matrix.backward_indices.shape[1]) == run
+    x, dy = torch.randn(tokens, fan_in), torch.randn(tokens, fan_out)
+    xd = x.to(DEV).to(BF16).requires_grad_(True)
+    y = layer(xd)
+    names, params = zip(*layer.named_parameters())
+    grads = torch.autograd.grad(y, [xd, *params], dy.to(DEV).to(BF16))
+    leaves = {n: p.detach().float().requires_grad_(True) for n, p in layer.named_parameters()}
+    xr = x.to(DEV).to(BF16).float().requires_grad_(True)
+    y_ref = xr @ _dense_from_native(leaves["matrix.weight"], matrix.backward_indices, fan_out).t() + leaves["bias"]
+    if lowrank_dim:
+        y_ref = y_ref + (xr @ leaves["matrix.lowrank_first"].t()) @ leaves["matrix.lowrank_second"].t()
+    ref = torch.autograd.grad(y_ref, [xr, *[leaves[n] for n in names]], dy.to(DEV).to(BF16).float())
+    assert_close(y, y_ref.detach(), BF16, "y")
+    assert_close(grads[0], ref[0], BF16, "dx")
+    for name, a, b in zip(names, grads[1:], ref[1:]):
+        assert_close(a, b, BF16, name)
+
+
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("tokens", [512, 300])
+def test_bf16_ffn_with_blocksparse_projections_in_runs(gated, tokens):
+    """LeanFFN whose up-projection is PixelFly stretched over a tall matrix (runs of output blocks with one list): plain GELU
+    takes the dense product's fused activation epilogue, GeGLU the product and the activation pass"""
+    torch.manual_seed(tokens + gated)
+    hidden, inter = 512, 2048
+    layout = "pixelfly(block_size=64, stretch=True)"
+    up = lt.GeneralizedLinear(lt.GeneralizedMatrix(hidden, inter * (2 if gated else 1), layout, 64))
+    down = lt.GeneralizedLinear(lt.GeneralizedMatrix(inter, hidden, layout, 64))
+    ffn = lt.LeanFFN(hidden, inter, gated=gated, i2h_proj=up, h2o_proj=down)
+    _randomise_small_vectors(ffn)
+    with torch.no_grad():
+        for t in (up.weight, down.weight, up.matrix.lowrank_first, up.matrix.lowrank_second, down.matrix.lowrank_first,
+                  down.matrix.lowrank_second):
+            t.normal_(std=0.05)
+    ffn = ffn.to(DEV).to(BF16)
+    x, dy = torch.randn(tokens, hidden), torch.randn(tokens, hidden)
+    _compare(ffn, x.to(BF16), dy.to(BF16), BF16)
