@@ -1309,6 +1309,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
 
   // ---- prologue: k-steps 0..2 (k-major: block 0 and the slot-0 halves of block 1) in flight and landed, first half of
   //      k-step 0 issued
+  LT_TILE_STAMP(6);
   if constexpr (A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J8{});
   if constexpr (B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J8{});
   if constexpr (!A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J4{});

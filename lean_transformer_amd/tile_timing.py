@@ -67,13 +67,14 @@ def main():
         ksteps = k // 32
         prologue, loop, epilogue = d[:, 1] - d[:, 0], d[:, 2] - d[:, 1], d[:, 3] - d[:, 2]
         first16 = (d[:, 7] - d[:, 1]).mean()
+        setup = (d[:, 6] - d[:, 0]).mean()  # launch to the first copy instruction: index arithmetic, bias loads
         clock = ((d[:, 3] - d[:, 0]) / ((d[:, 5] - d[:, 4]) * 10.0)).mean()
         span = (d[:, 5].max() - d[:, 4].min()) / 100.0
         per_tile = (prologue + loop + epilogue).mean()
         total_ticks += per_tile * len(d)
         total_ideal += ksteps * 1024.0 * len(d)
         print(f"{label:28s} tiles {len(d):5d}  span {span:7.1f} us  ticks/tile {per_tile:9.0f}  ideal {ksteps * 1024:8d} "
-              f"({ksteps * 1024 / per_tile:.3f})  prologue {prologue.mean():6.0f}  loop {loop.mean():9.0f} = "
+              f"({ksteps * 1024 / per_tile:.3f})  prologue {prologue.mean():6.0f} (of which before the first copy {setup:5.0f})  loop {loop.mean():9.0f} = "
               f"{loop.mean() / ksteps:6.1f}/k-step (first 16: {first16 / 16:6.1f}, rest: "
               f"{(loop.mean() - first16) / (ksteps - 16):6.1f})  epilogue {epilogue.mean():6.0f} (max {epilogue.max():6d})  "
               f"clock {clock:.3f} GHz")
