@@ -255,3 +255,20 @@ def test_native_and_block_list_weight_orders():
         assert torch.equal(lt.block_list_to_native(blocks[perm], coords[perm], m.backward_indices), w)
     with pytest.raises(ValueError):
         lt.block_list_to_native(blocks, coords.flip(1), m.backward_indices[:, :1])
+
+
+def test_shared_list_run_of_pixelfly_layouts():
+    """runs of consecutive output blocks with one list of input blocks: stretched PixelFly on a tall matrix repeats every list
+    out_blocks / in_blocks times, the tiled form and square matrices have none; the cached value follows in-place changes"""
+    from lean_transformer_amd.blocksparse.linear import shared_list_run
+    for out_f, in_f, stretch, expected in [(4096, 1024, True, 4), (4096, 512, True, 8), (4096, 1024, False, 1),
+                                           (1024, 1024, True, 1), (1024, 4096, True, 1)]:
+        layout = lt.get_blocksparse_layout(out_f, in_f, f"pixelfly(block_size=64, stretch={stretch})")
+        forward_indices, backward_indices = lt.get_indices_from_layout(layout)
+        assert shared_list_run(forward_indices, backward_indices.shape[1]) == expected, (out_f, in_f, stretch)
+    layout = lt.get_blocksparse_layout(4096, 1024, "pixelfly(block_size=64, stretch=True)")
+    forward_indices, backward_indices = lt.get_indices_from_layout(layout)
+    per_in = backward_indices.shape[1]
+    assert shared_list_run(forward_indices, per_in) == 4
+    forward_indices[1] = forward_indices[8]  # output block 1 now reads other input blocks than 0, 2 and 3
+    assert shared_list_run(forward_indices, per_in) == 1
