@@ -301,3 +301,29 @@ def test_bf16_ffn_with_blocksparse_projections_in_runs(gated, tokens):
     ffn = ffn.to(DEV).to(BF16)
     x, dy = torch.randn(tokens, hidden), torch.randn(tokens, hidden)
     _compare(ffn, x.to(BF16), dy.to(BF16), BF16)
+
+
+@pytest.mark.parametrize("sparse", [False, True])
+def test_repeated_steps_are_bitwise_identical(sparse):
+    """no kernel on the path sums in an order that depends on scheduling (split reductions are summed in slice order, column
+    sums per fixed row slices, no atomics): the same step twice gives the same bits in y and in every gradient"""
+    torch.manual_seed(5)
+    hidden, inter = 512, 2048
+    if sparse:
+        layout = "pixelfly(block_size=64, stretch=True)"
+        up = lt.GeneralizedLinear(lt.GeneralizedMatrix(hidden, 2 * inter, layout, 64))
+        down = lt.GeneralizedLinear(lt.GeneralizedMatrix(inter, hidden, layout, 64))
+        ffn = lt.LeanFFN(hidden, inter, gated=True, i2h_proj=up, h2o_proj=down, dropout=0.1)
+    else:
+        ffn = lt.LeanFFN(hidden, inter, gated=True, dropout=0.1)
+    ffn = ffn.to(DEV).to(BF16).train()
+    x = torch.randn(1024, hidden, device=DEV, dtype=BF16, requires_grad=True)
+    dy = torch.randn(1024, hidden, device=DEV, dtype=BF16)
+    params = list(ffn.parameters())
+    runs = []
+    for _ in range(2):
+        torch.manual_seed(11)  # same dropout stream
+        y = ffn(x)
+        runs.append([y.detach().clone()] + [g.clone() for g in torch.autograd.grad(y, [x, *params], dy)])
+    for a, b in zip(*runs):
+        assert torch.equal(a, b)
