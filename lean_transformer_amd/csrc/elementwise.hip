@@ -28,58 +28,76 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(int64_t T, int H, float eps
   const float inv_h = 1.0f / (float)H;
   float mean, rstd;
   if (vec) {
-    float v[MAXV][4];
-    float s = 0.f;
+    // W elements per lane per piece: 8 where the row length allows it, so that a bf16 output leaves in 16-byte stores
+    auto row_in_registers = [&](auto W_c) {
+      constexpr int W = decltype(W_c)::value, PIECES = MAXV * 4 / W;
+      float v[PIECES][W];
+      float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < MAXV; i++) {
-      const int c = (i * 64 + lane) * 4;
-      if (c < H) {
-        load4(xr + c, v[i]);
-        s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
-      }
-    }
-    mean = wave_sum(s) * inv_h;
-    float q = 0.f;
-#pragma unroll
-    for (int i = 0; i < MAXV; i++) {
-      const int c = (i * 64 + lane) * 4;
-      if (c < H) {
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const float d = v[i][e] - mean;
-          q += d * d;
-        }
-      }
-    }
-    rstd = 1.0f / sqrtf(wave_sum(q) * inv_h + eps);
-    if (y) {
-#pragma unroll
-      for (int i = 0; i < MAXV; i++) {
-        const int c = (i * 64 + lane) * 4;
+      for (int i = 0; i < PIECES; i++) {
+        const int c = (i * 64 + lane) * W;
         if (c < H) {
-          float wv[4], bv[4], o[4];
-          load4(w + c, wv);
-          load4(b + c, bv);
+          if constexpr (W == 8) load8(xr + c, v[i]);
+          else load4(xr + c, v[i]);
 #pragma unroll
-          for (int e = 0; e < 4; e++) o[e] = (v[i][e] - mean) * rstd * wv[e] + bv[e];
-          if constexpr (TAIL) {
-            if (drop.p > 0.f) {
-              bool keep[4];
-              dropout_keep4(drop, row * H + c, keep);
-#pragma unroll
-              for (int e = 0; e < 4; e++) o[e] = keep[e] ? o[e] * drop.scale : 0.f;
-            }
-            if (residual) {
-              float rv[4];
-              load4(residual + row * H + c, rv);
-#pragma unroll
-              for (int e = 0; e < 4; e++) o[e] += rv[e];
-            }
-          }
-          store4(y + row * H + c, o);
+          for (int e = 0; e < W; e++) s += v[i][e];
         }
       }
-    }
+      mean = wave_sum(s) * inv_h;
+      float q = 0.f;
+#pragma unroll
+      for (int i = 0; i < PIECES; i++) {
+        const int c = (i * 64 + lane) * W;
+        if (c < H) {
+#pragma unroll
+          for (int e = 0; e < W; e++) {
+            const float d = v[i][e] - mean;
+            q += d * d;
+          }
+        }
+      }
+      rstd = 1.0f / sqrtf(wave_sum(q) * inv_h + eps);
+      if (y) {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+          const int c = (i * 64 + lane) * W;
+          if (c < H) {
+            float wv[W], bv[W], o[W];
+            if constexpr (W == 8) {
+              load8(w + c, wv);
+              load8(b + c, bv);
+            } else {
+              load4(w + c, wv);
+              load4(b + c, bv);
+            }
+#pragma unroll
+            for (int e = 0; e < W; e++) o[e] = (v[i][e] - mean) * rstd * wv[e] + bv[e];
+            if constexpr (TAIL) {
+              if (drop.p > 0.f) {
+#pragma unroll
+                for (int h = 0; h < W / 4; h++) {
+                  bool keep[4];
+                  dropout_keep4(drop, row * H + c + 4 * h, keep);
+#pragma unroll
+                  for (int e = 0; e < 4; e++) o[4 * h + e] = keep[e] ? o[4 * h + e] * drop.scale : 0.f;
+                }
+              }
+              if (residual) {
+                float rv[W];
+                if constexpr (W == 8) load8(residual + row * H + c, rv);
+                else load4(residual + row * H + c, rv);
+#pragma unroll
+                for (int e = 0; e < W; e++) o[e] += rv[e];
+              }
+            }
+            if constexpr (W == 8) store8(y + row * H + c, o);
+            else store4(y + row * H + c, o);
+          }
+        }
+      }
+    };
+    if (vec == 2) row_in_registers(std::integral_constant<int, 8>{});
+    else row_in_registers(std::integral_constant<int, 4>{});
   } else {
     float s = 0.f;
     for (int c = lane; c < H; c += 64) s += ldf(xr, c);
@@ -564,8 +582,9 @@ int lt_ln_forward(int64_t T, int H, float eps, int x_dtype, const void* x, const
   LT_REQUIRE(T > 0 && H > 0 && x, LT_ERR_BAD_ARG, "layernorm: bad arguments");
   LT_REQUIRE(!y || (w && b), LT_ERR_BAD_ARG, "layernorm: weight and bias are required when an output is requested");
   // rows are held in registers and moved 4 elements at a time when the size and every pointer allow it
-  const int vec = (H & 3) == 0 && H <= 64 * 4 * LN_MAXV && lt_aligned(x, 16) && (!y || lt_aligned(y, 16)) &&
-                  (!w || lt_aligned(w, 16)) && (!b || lt_aligned(b, 16)) && (!residual || lt_aligned(residual, 16));
+  int vec = (H & 3) == 0 && H <= 64 * 4 * LN_MAXV && lt_aligned(x, 16) && (!y || lt_aligned(y, 16)) &&
+            (!w || lt_aligned(w, 16)) && (!b || lt_aligned(b, 16)) && (!residual || lt_aligned(residual, 16));
+  if (vec && (H & 7) == 0) vec = 2;  // 8 elements per lane per piece: 16-byte stores of a bf16 output
   dim3 grid(blocks_for(T, 4)), block(256);
   DropoutParams d = drop ? *drop : make_dropout(0.f, 0, 0);
   LtProfileScope scope(tail ? "layernorm_fwd_tail" : (y ? "layernorm_fwd" : "layernorm_stats"), 0.0,
