@@ -1053,27 +1053,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   const int64_t m0 = (int64_t)tm * BM;
   const int64_t n0 = (int64_t)tn * (gated ? BN / 2 : BN);
 
-  // The accumulators start at the bias of their column (a lane holds one column per 32-wide block), so no epilogue has to
-  // add it.  Gated forward: blocks 0, 1 of a wavefront are gate columns, 2, 3 the matching linear columns.
-  float bias0[FN];
-#pragma unroll
-  for (int j = 0; j < FN; j++) {
-    bias0[j] = 0.f;
-    if (p.epi.bias) {
-      // columns past N (a tile that sticks out) take the last column's bias and are never written
-      const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) +
-                                      min(n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31), p.N - 1)
-                                : min(n0 + wn * WTN + j * 32 + (lane & 31), p.N - 1);
-      bias0[j] = p.epi.bias[col];
-    }
-  }
-  f32x16 acc[FM][FN];
-#pragma unroll
-  for (int i = 0; i < FM; i++)
-#pragma unroll
-    for (int j = 0; j < FN; j++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = bias0[j];
+  f32x16 acc[FM][FN];  // initialised in the prologue, after the first copies have gone out
 
   const int kt_all = (int)((p.K[0] + DK - 1) / DK) + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
   // split-k (one k-segment only): this workgroup walks k-steps [kt_begin, kt_begin + kt_total) of kt_all; the slices are
@@ -1323,6 +1303,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
     if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2, J0{}, J4{});
     if constexpr (N_KM > 0) copy_block_halves(Ragged{}, std::integral_constant<int, 0>{}, P2{}, 2);
   }
+  // The accumulators start at the bias of their column (a lane holds one column per 32-wide block), so no epilogue has to
+  // add it.  The bias loads wait behind the first copies rather than in front of them.  Gated forward: blocks 0, 1 of a
+  // wavefront are gate columns, 2, 3 the matching linear columns.
+  float bias0[FN];
+#pragma unroll
+  for (int j = 0; j < FN; j++) {
+    bias0[j] = 0.f;
+    if (p.epi.bias) {
+      // columns past N (a tile that sticks out) take the last column's bias and are never written
+      const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) +
+                                      min(n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31), p.N - 1)
+                                : min(n0 + wn * WTN + j * 32 + (lane & 31), p.N - 1);
+      bias0[j] = p.epi.bias[col];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < FM; i++)
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = bias0[j];
   wait_copies_and_barrier<0>();
   LT_TILE_STAMP(1);
   load_frags(P0{}, 0, af[0], bfr[0]);
