@@ -16,11 +16,20 @@ def _step(ffn, x, dy, params):
     return (y, *torch.autograd.grad(y, [x, *params], dy))
 
 
-@pytest.mark.parametrize("hidden,inter,tokens,dtype", [(512, 1024, 300, torch.bfloat16), (256, 4096, 200, torch.bfloat16),
-                                                       (192, 320, 130, torch.float32)])
-def test_ffn_step_replays_from_a_graph(hidden, inter, tokens, dtype):
+@pytest.mark.parametrize("hidden,inter,tokens,dtype,layout", [
+    (512, 1024, 300, torch.bfloat16, None), (256, 4096, 200, torch.bfloat16, None), (192, 320, 130, torch.float32, None),
+    # block-sparse projections: the walks, and (stretched PixelFly) the dense products over gathered blocks with their split
+    # rank-64 GEMMs; the warm-up steps settle the once-per-index-tensor host check of the layout's structure before capture
+    (512, 2048, 512, torch.bfloat16, "pixelfly(block_size=64, stretch=True)"),
+    (512, 2048, 300, torch.bfloat16, "pixelfly(block_size=64, stretch=False)")])
+def test_ffn_step_replays_from_a_graph(hidden, inter, tokens, dtype, layout):
     torch.manual_seed(hidden + tokens)
-    ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5)
+    if layout is None:
+        ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5)
+    else:
+        up = lt.GeneralizedLinear(lt.GeneralizedMatrix(hidden, 2 * inter, layout, 64))
+        down = lt.GeneralizedLinear(lt.GeneralizedMatrix(inter, hidden, layout, 64))
+        ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5, i2h_proj=up, h2o_proj=down)
     with torch.no_grad():
         ffn.i2h_proj.bias.normal_(std=0.1)
         ffn.h2o_proj.bias.normal_(std=0.1)
