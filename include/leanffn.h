@@ -57,8 +57,10 @@ typedef struct lt_linear {
   int32_t blocks_per_out; /* K: active blocks per output block row */
   int32_t blocks_per_in;  /* A: active blocks per input block column */
   int32_t out_group;      /* sparse: every aligned run of this many consecutive output blocks has the same list of input
-                             blocks (PixelFly with stretch=True on a tall matrix: out_blocks / in_blocks).  A promise by the
-                             caller that only selects a faster weight-gradient kernel; 0 or 1 when not known. */
+                             blocks, and under each of them the run's weight blocks are adjacent (forward_indices of output
+                             block ob0 + j = those of ob0, + j).  PixelFly with stretch=True on a tall matrix: out_blocks /
+                             in_blocks.  A promise by the caller that only selects faster forward and weight-gradient
+                             kernels; 0 or 1 when not known. */
   int32_t reserved;       /* 0 */
 } lt_linear;
 

@@ -152,7 +152,12 @@ def shared_list_run(forward_indices: torch.Tensor, blocks_per_in: int) -> int:
     run, n_out = 1, lists.shape[0]
     while n_out % (2 * run) == 0:
         grouped = lists.reshape(n_out // (2 * run), 2 * run, -1)
-        if not bool((grouped == grouped[:, :1]).all()):
+        # ... and the run's weight blocks must sit next to each other under every input block of the list (they do when the
+        # index tables list active blocks in ascending order, as get_indices_from_layout builds them): the kernels read them
+        # as one matrix
+        flat = forward_indices.reshape(n_out // (2 * run), 2 * run, -1)
+        step = torch.arange(2 * run, device=flat.device, dtype=flat.dtype)[None, :, None]
+        if not bool(((grouped == grouped[:, :1]) & (flat == flat[:, :1] + step)).all()):
             break
         run *= 2
     forward_indices._lt_shared_list_run = ((forward_indices._version, blocks_per_in), run)
