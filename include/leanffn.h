@@ -39,7 +39,28 @@ typedef enum lt_status {
 
 typedef enum lt_dtype { LT_F32 = 0, LT_BF16 = 1 } lt_dtype;
 
-typedef enum lt_act { LT_ACT_GELU_FUSED = 0, LT_ACT_GELU = 1, LT_ACT_RELU = 2, LT_ACT_SILU = 3 } lt_act;
+/* Activations evaluated in registers, value and derivative: the reference's gelu_fused (tanh form, lean_transformer/utils.py:24-38)
+ * and the closed-form entries of transformers.activations.ACT2FN, the table the reference's ACT2FN extends (utils.py:80).
+ * LT_ACT_GELU is the erf form; leaky_relu has slope 0.01.  Entries with learned parameters (prelu, xielu) have no kind. */
+typedef enum lt_act {
+  LT_ACT_GELU_FUSED = 0,
+  LT_ACT_GELU = 1,
+  LT_ACT_RELU = 2,
+  LT_ACT_SILU = 3,
+  LT_ACT_QUICK_GELU = 4,
+  LT_ACT_GELU_10 = 5,
+  LT_ACT_RELU6 = 6,
+  LT_ACT_RELU2 = 7,
+  LT_ACT_LEAKY_RELU = 8,
+  LT_ACT_MISH = 9,
+  LT_ACT_SIGMOID = 10,
+  LT_ACT_TANH = 11,
+  LT_ACT_LINEAR = 12,
+  LT_ACT_HARDSWISH = 13,
+  LT_ACT_LAPLACE = 14,
+  LT_ACT_SQRT_SOFTPLUS = 15,
+  LT_ACT_COUNT = 16
+} lt_act;
 
 /* One projection in the reference's "generalized linear" form: main weight (dense or native block-sparse), optional bias,
  * optional low-rank pair.  Weights and low-rank factors are in the compute dtype; the bias is always fp32. */

@@ -260,7 +260,7 @@ int check_ffn_desc(const lt_ffn_desc* d) {
   LT_TRY(check_dtype(d->compute_dtype, "ffn compute_dtype"));
   // the LayerNorm kernels hold a row in registers (backward has no strided variant): refuse wider rows before any work
   LT_REQUIRE(d->hidden <= 8192, LT_ERR_UNSUPPORTED, "ffn: hidden size %d exceeds 8192, the widest row the LayerNorm kernels take", d->hidden);
-  LT_REQUIRE(d->act >= LT_ACT_GELU_FUSED && d->act <= LT_ACT_SILU, LT_ERR_UNSUPPORTED, "ffn: unknown activation %d", d->act);
+  LT_REQUIRE(d->act >= 0 && d->act < LT_ACT_COUNT, LT_ERR_UNSUPPORTED, "ffn: unknown activation %d", d->act);
   LT_REQUIRE(d->ln_weight && d->ln_bias, LT_ERR_BAD_ARG, "ffn: LayerNorm parameters missing");
   LT_REQUIRE((d->post_ln_weight == nullptr) == (d->post_ln_bias == nullptr), LT_ERR_BAD_ARG, "ffn: post-LN needs weight and bias");
   LT_REQUIRE(d->dropout_p >= 0.f && d->dropout_p < 1.f, LT_ERR_BAD_ARG, "ffn: dropout %f outside [0, 1)", d->dropout_p);
@@ -570,14 +570,14 @@ extern "C" int lt_layernorm_backward(int64_t tokens, int32_t hidden, int32_t x_d
 extern "C" int lt_activation_forward(int64_t tokens, int32_t intermediate, int32_t gated, int32_t act, int32_t dtype,
                                      const void* pre, void* hid, void* stream) {
   LT_TRY(check_dtype(dtype, "activation"));
-  LT_REQUIRE(act >= LT_ACT_GELU_FUSED && act <= LT_ACT_SILU, LT_ERR_UNSUPPORTED, "unknown activation %d", act);
+  LT_REQUIRE(act >= 0 && act < LT_ACT_COUNT, LT_ERR_UNSUPPORTED, "unknown activation %d", act);
   return lt_act_forward(tokens, intermediate, gated, act, dtype, pre, hid, (hipStream_t)stream);
 }
 
 extern "C" int lt_activation_backward(int64_t tokens, int32_t intermediate, int32_t gated, int32_t act, int32_t dtype,
                                       const void* pre, const void* d_hid, void* d_pre, void* stream) {
   LT_TRY(check_dtype(dtype, "activation backward"));
-  LT_REQUIRE(act >= LT_ACT_GELU_FUSED && act <= LT_ACT_SILU, LT_ERR_UNSUPPORTED, "unknown activation %d", act);
+  LT_REQUIRE(act >= 0 && act < LT_ACT_COUNT, LT_ERR_UNSUPPORTED, "unknown activation %d", act);
   return lt_act_backward(tokens, intermediate, gated, act, dtype, pre, d_hid, d_pre, (hipStream_t)stream);
 }
 

@@ -188,10 +188,79 @@ template <bool PRECISE> __device__ __forceinline__ void act_eval(int act, float 
       value = x > 0.0f ? x : 0.0f;
       deriv = x > 0.0f ? 1.0f : 0.0f;
       break;
-    default: {  // LT_ACT_SILU
+    case LT_ACT_SILU: {
       float s = lt_sigmoid<PRECISE>(x);
       value = x * s;
       deriv = s * (1.0f + x * (1.0f - s));
+      break;
+    }
+    // The remaining closed-form entries of the Hugging Face activation table (the table the reference extends,
+    // lean_transformer/utils.py:80).  They run through the general epilogue strips; libm-grade functions throughout.
+    case LT_ACT_QUICK_GELU: {
+      float s = lt_sigmoid<PRECISE>(1.702f * x);
+      value = x * s;
+      deriv = s + 1.702f * x * s * (1.0f - s);
+      break;
+    }
+    case LT_ACT_GELU_10: {  // clip(gelu(x), -10, 10): the clip passes gradients where gelu(x) lies inside the interval
+      float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752f));
+      float g = x * cdf;
+      value = fminf(fmaxf(g, -10.0f), 10.0f);
+      deriv = (g >= -10.0f && g <= 10.0f) ? cdf + x * expf(-0.5f * x * x) * 0.39894228040143268f : 0.0f;
+      break;
+    }
+    case LT_ACT_RELU6:
+      value = fminf(fmaxf(x, 0.0f), 6.0f);
+      deriv = (x > 0.0f && x < 6.0f) ? 1.0f : 0.0f;
+      break;
+    case LT_ACT_RELU2: {
+      float r = x > 0.0f ? x : 0.0f;
+      value = r * r;
+      deriv = 2.0f * r;
+      break;
+    }
+    case LT_ACT_LEAKY_RELU:  // negative slope 0.01 (torch.nn.LeakyReLU's default, the table's entry)
+      value = x > 0.0f ? x : 0.01f * x;
+      deriv = x > 0.0f ? 1.0f : 0.01f;
+      break;
+    case LT_ACT_MISH: {  // x tanh(softplus(x)); softplus(x) = x beyond 20 like torch's
+      float sp = x > 20.0f ? x : log1pf(expf(x));
+      float t = tanhf(sp);
+      value = x * t;
+      deriv = t + x * (1.0f - t * t) * lt_sigmoid<true>(x);
+      break;
+    }
+    case LT_ACT_SIGMOID: {
+      float s = lt_sigmoid<true>(x);
+      value = s;
+      deriv = s * (1.0f - s);
+      break;
+    }
+    case LT_ACT_TANH: {
+      float t = tanhf(x);
+      value = t;
+      deriv = 1.0f - t * t;
+      break;
+    }
+    case LT_ACT_LINEAR:
+      value = x;
+      deriv = 1.0f;
+      break;
+    case LT_ACT_HARDSWISH:
+      value = x * fminf(fmaxf(x + 3.0f, 0.0f), 6.0f) * (1.0f / 6.0f);
+      deriv = x < -3.0f ? 0.0f : (x <= 3.0f ? x * (1.0f / 3.0f) + 0.5f : 1.0f);
+      break;
+    case LT_ACT_LAPLACE: {  // 0.5 (1 + erf((x - mu) / (sigma sqrt 2))), mu = 0.707107, sigma = 0.282095
+      const float inv = 1.0f / (0.282095f * 1.41421356237f);
+      float z = (x - 0.707107f) * inv;
+      value = 0.5f * (1.0f + erff(z));
+      deriv = expf(-z * z) * inv * 0.56418958354775629f;  // 1 / sqrt(pi)
+      break;
+    }
+    default: {  // LT_ACT_SQRT_SOFTPLUS
+      float sp = x > 20.0f ? x : log1pf(expf(x));
+      value = sqrtf(sp);
+      deriv = value > 0.0f ? lt_sigmoid<true>(x) / (2.0f * value) : 0.0f;  // softplus underflows to 0 far in the negative tail
       break;
     }
   }

@@ -34,6 +34,15 @@ def gelu_fused_grad(grad_output: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     return jac * grad_output
 
 
+# The closed-form entries of transformers.activations.ACT2FN (the table the reference extends at utils.py:80; transformers
+# is a third-party dependency of the reference, not part of its checkout).  Restated from the published definitions of each
+# function; tests/test_oracle.py pins every value against the installed transformers table and every derivative against
+# fp64 autograd of the value.
+LAPLACE_MU, LAPLACE_SIGMA = 0.707107, 0.282095
+ACT_NAMES = ("gelu_fused", "gelu", "relu", "silu", "quick_gelu", "gelu_10", "relu6", "relu2", "leaky_relu", "mish", "sigmoid",
+             "tanh", "linear", "hardswish", "laplace", "sqrtsoftplus")
+
+
 def act_forward(kind: str, x: torch.Tensor) -> torch.Tensor:
     if kind == "gelu_fused":
         return gelu_fused(x)
@@ -43,22 +52,84 @@ def act_forward(kind: str, x: torch.Tensor) -> torch.Tensor:
         return F.relu(x)
     if kind == "silu":
         return F.silu(x)
+    if kind == "quick_gelu":
+        return x * torch.sigmoid(1.702 * x)
+    if kind == "gelu_10":
+        return torch.clip(F.gelu(x), -10, 10)
+    if kind == "relu6":
+        return torch.clamp(x, 0, 6)
+    if kind == "relu2":
+        return torch.square(F.relu(x))
+    if kind == "leaky_relu":
+        return torch.where(x > 0, x, 0.01 * x)
+    if kind == "mish":
+        return x * torch.tanh(F.softplus(x))
+    if kind == "sigmoid":
+        return torch.sigmoid(x)
+    if kind == "tanh":
+        return torch.tanh(x)
+    if kind == "linear":
+        return x
+    if kind == "hardswish":
+        return x * torch.clamp(x + 3, 0, 6) / 6
+    if kind == "laplace":
+        return 0.5 * (1.0 + torch.erf((x - LAPLACE_MU) / (LAPLACE_SIGMA * 2.0 ** 0.5)))
+    if kind == "sqrtsoftplus":
+        return torch.sqrt(F.softplus(x))
+    raise ValueError(kind)
+
+
+def act_derivative(kind: str, x: torch.Tensor) -> torch.Tensor:
+    """d act(x) / dx, element-wise, written out by hand (at a kink: the one-sided value autograd takes)"""
+    one, zero = torch.ones_like(x), torch.zeros_like(x)
+    if kind == "gelu_fused":
+        return gelu_fused_grad(one, x)
+    if kind in ("gelu", "gelu_10"):
+        cdf = 0.5 * (1 + torch.erf(x * 0.7071067811865476))
+        pdf = torch.exp(-0.5 * x * x) * 0.3989422804014327
+        jac = cdf + x * pdf
+        if kind == "gelu_10":  # the clip passes gradients where its input lies inside [-10, 10]
+            g = x * cdf
+            jac = torch.where((g >= -10) & (g <= 10), jac, zero)
+        return jac
+    if kind == "relu":
+        return (x > 0).to(x.dtype)
+    if kind == "silu":
+        s = torch.sigmoid(x)
+        return s * (1 + x * (1 - s))
+    if kind == "quick_gelu":
+        s = torch.sigmoid(1.702 * x)
+        return s + 1.702 * x * s * (1 - s)
+    if kind == "relu6":
+        return ((x > 0) & (x < 6)).to(x.dtype)
+    if kind == "relu2":
+        return 2 * F.relu(x)
+    if kind == "leaky_relu":
+        return torch.where(x > 0, one, 0.01 * one)
+    if kind == "mish":
+        t = torch.tanh(F.softplus(x))
+        return t + x * (1 - t * t) * torch.sigmoid(x)
+    if kind == "sigmoid":
+        s = torch.sigmoid(x)
+        return s * (1 - s)
+    if kind == "tanh":
+        t = torch.tanh(x)
+        return 1 - t * t
+    if kind == "linear":
+        return one
+    if kind == "hardswish":
+        return torch.where(x < -3, zero, torch.where(x <= 3, x / 3 + 0.5, one))
+    if kind == "laplace":
+        scale = LAPLACE_SIGMA * 2.0 ** 0.5
+        z = (x - LAPLACE_MU) / scale
+        return torch.exp(-z * z) / (scale * 3.141592653589793 ** 0.5)
+    if kind == "sqrtsoftplus":
+        return torch.sigmoid(x) / (2 * torch.sqrt(F.softplus(x)))
     raise ValueError(kind)
 
 
 def act_backward(kind: str, grad: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-    if kind == "gelu_fused":
-        return gelu_fused_grad(grad, x)
-    if kind == "gelu":
-        cdf = 0.5 * (1 + torch.erf(x * 0.7071067811865476))
-        pdf = torch.exp(-0.5 * x * x) * 0.3989422804014327
-        return grad * (cdf + x * pdf)
-    if kind == "relu":
-        return grad * (x > 0).to(grad.dtype)
-    if kind == "silu":
-        s = torch.sigmoid(x)
-        return grad * (s * (1 + x * (1 - s)))
-    raise ValueError(kind)
+    return grad * act_derivative(kind, x)
 
 
 @dataclass

@@ -30,12 +30,18 @@ def _randomise_small_vectors(ffn, seed=0):
                 proj.bias.copy_(torch.randn(proj.bias.shape, generator=g) * 0.1)
 
 
-@pytest.mark.parametrize("act", ["gelu", "relu", "silu"])
-@pytest.mark.parametrize("gated", [False, True])
-@pytest.mark.parametrize("tokens", [512, 300])
+KINKED = ("relu", "relu6", "leaky_relu", "hardswish")  # derivative jumps: see the docstring below
+OTHER_ACTS = [(a, g, t) for a in ("gelu", "relu", "silu") for g in (False, True) for t in (512, 300)] + [
+    (a, i % 2 == 0, 300 if i % 3 == 0 else 512) for i, a in enumerate(
+        ("quick_gelu", "gelu_10", "relu6", "relu2", "leaky_relu", "mish", "sigmoid", "tanh", "linear", "hardswish", "laplace",
+         "sqrtsoftplus", "gelu_accurate", "gelu_fast"))]
+
+
+@pytest.mark.parametrize("act,gated,tokens", OTHER_ACTS)
 def test_bf16_other_activations_take_the_general_epilogue_strips(act, gated, tokens):
     """the straight-line strips are compiled for the tanh GELU; every other activation goes through the strips that choose
-    per row (forward activation epilogue, backward d-activation epilogue with its fused column sums).  relu's derivative
+    per row (forward activation epilogue, backward d-activation epilogue with its fused column sums).  Every closed-form
+    entry of the Hugging Face table has a row.  The derivative of relu (and of relu6, leaky_relu, hardswish)
     jumps at 0, so its gradients depend on the sign of the pre-activation as stored (bf16): the oracle is asked to round
     where the bf16 path stores (LayerNorm output, pre-activation, activation output), which is what the reference does
     under bf16 autocast; the smooth activations are compared with the unrounded fp32 oracle like everywhere else."""
@@ -43,7 +49,7 @@ def test_bf16_other_activations_take_the_general_epilogue_strips(act, gated, tok
     ffn = lt.LeanFFN(512, 1024, activation=ACT2FN[act], gated=gated, layer_norm_eps=1e-5)
     _randomise_small_vectors(ffn)
     ffn = ffn.to(DEV).to(BF16)
-    _compare(ffn, torch.randn(tokens, 512), torch.randn(tokens, 512), BF16, bf16_rounding=(act == "relu"))
+    _compare(ffn, torch.randn(tokens, 512), torch.randn(tokens, 512), BF16, bf16_rounding=(act in KINKED))
 
 
 @pytest.mark.parametrize("io_dtype", [torch.float32, BF16])

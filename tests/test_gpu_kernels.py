@@ -160,14 +160,17 @@ def test_layernorm_backward(tokens, hidden, x_dtype, dy_dtype, dx_dtype, with_re
     assert_close(db, br.grad.float(), torch.float32, "dbias")
 
 
-@pytest.mark.parametrize("act", ["gelu_fused", "gelu", "relu", "silu"])
+@pytest.mark.parametrize("act", offn.ACT_NAMES)
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_activation_forward_backward(act, gated, dtype):
+    """every kernel-side activation, value and derivative, against fp64 autograd of the oracle's value on the same stored
+    pre-activations (so the kinks of the piecewise ones fall on the same side)"""
     from lean_transformer_amd.utils import ACT_KINDS
     tokens, inter = 33, 70
     g = torch.Generator().manual_seed(5)
     pre = (torch.randn(tokens, 2 * inter if gated else inter, generator=g) * 3).to(dtype)
+    pre[0, :6] = torch.tensor([11.0, -11.0, 25.0, -25.0, 6.5, -3.5]).to(dtype)  # beyond gelu_10's clip, softplus' switch, the kinks
     dh = torch.randn(tokens, inter, generator=g).to(dtype)
     pr = pre.double().requires_grad_(True)
     href = offn.apply_activation(pr, act, gated)

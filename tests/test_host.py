@@ -130,8 +130,9 @@ def test_activation_mapping():
     assert activation_kind(ACT2FN["gelu_new"]) == "gelu_fused"
     assert activation_kind(ACT2FN["relu"]) == "relu" and activation_kind(ACT2FN["swish"]) == "silu"
     assert activation_kind(torch.nn.functional.gelu) == "gelu" and activation_kind(nn.GELU(approximate="tanh")) == "gelu_fused"
+    assert activation_kind(torch.sigmoid) == "sigmoid" and activation_kind(nn.LeakyReLU()) == "leaky_relu"
     with pytest.raises(NotImplementedError):
-        activation_kind(torch.sigmoid)
+        activation_kind(torch.exp)
     x = torch.linspace(-5, 5, 1000)
     assert (ACT2FN["gelu_fused"](x) - torch.nn.functional.gelu(x)).abs().max().item() <= 5e-4  # reference tests/test_utils.py:25-29
     assert torch.allclose(ACT2FN["gelu_fused"](x), offn.gelu_fused(x))

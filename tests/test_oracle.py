@@ -119,12 +119,52 @@ def test_gelu_fused_close_to_erf_gelu():
     assert (offn.gelu_fused(x) - F.gelu(x)).abs().max().item() <= 5e-4
 
 
-@pytest.mark.parametrize("kind", ["gelu_fused", "gelu", "relu", "silu"])
+@pytest.mark.parametrize("kind", offn.ACT_NAMES)
 def test_activation_grad_is_autograd_of_forward(kind):
-    x = torch.linspace(-6, 6, 2001, dtype=torch.float64)[1:-1:2].clone().requires_grad_(True)  # avoids relu's kink at 0
+    # an even count of points over (-12, 12) misses the kinks at 0, +-3 and 6; gelu_10's clip at gelu(x) = 10 lies inside
+    x = torch.linspace(-12, 12, 4001, dtype=torch.float64)[1:-1:2].clone().requires_grad_(True)
     g = torch.randn(x.shape, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
     (auto,) = torch.autograd.grad(offn.act_forward(kind, x), x, g)
     assert torch.allclose(offn.act_backward(kind, g, x.detach()), auto, rtol=1e-6, atol=1e-7)
+    if kind == "gelu_10":
+        assert (offn.act_derivative(kind, x.detach())[x.detach() > 10.5] == 0).all()  # the clip is exercised
+
+
+HF_NAMES = {  # entry of transformers.activations.ACT2FN -> the oracle's (and the kernels') activation
+    "gelu": "gelu", "gelu_python": "gelu", "gelu_new": "gelu_fused", "gelu_fast": "gelu_fused", "gelu_pytorch_tanh": "gelu_fused",
+    "gelu_python_tanh": "gelu_fused", "gelu_accurate": "gelu_fused", "relu": "relu", "silu": "silu", "swish": "silu",
+    "quick_gelu": "quick_gelu", "gelu_10": "gelu_10", "relu6": "relu6", "relu2": "relu2", "leaky_relu": "leaky_relu",
+    "mish": "mish", "sigmoid": "sigmoid", "tanh": "tanh", "linear": "linear", "hardswish": "hardswish", "laplace": "laplace",
+    "sqrtsoftplus": "sqrtsoftplus"}
+
+
+@pytest.mark.parametrize("name", sorted(HF_NAMES))
+def test_activation_values_match_the_huggingface_table(name):
+    """The reference's ACT2FN is transformers' table plus gelu_fused (utils.py:80): every closed-form entry the installed
+    transformers has must equal the oracle's restatement (the tanh-form GELUs up to the digits of sqrt(2 / pi) the reference
+    truncates: 3e-10), and the package's own table must name the same kernel-side activation for it."""
+    hf = pytest.importorskip("transformers.activations").ACT2FN
+    if name not in hf:
+        pytest.skip(f"this transformers has no {name}")
+    from lean_transformer_amd.utils import ACT2FN, activation_kind
+    kind = HF_NAMES[name]
+    x = torch.linspace(-12, 12, 4001, dtype=torch.float64)
+    assert (offn.act_forward(kind, x) - hf[name](x)).abs().max().item() <= (1e-9 if kind == "gelu_fused" else 1e-14)
+    assert activation_kind(hf[name]) == kind and activation_kind(ACT2FN[name]) == kind
+    assert (ACT2FN[name](x) - hf[name](x)).abs().max().item() <= 1e-9
+
+
+def test_activations_with_learned_parameters_are_refused():
+    hf = pytest.importorskip("transformers.activations").ACT2FN
+    from lean_transformer_amd.utils import activation_kind
+    for name in ("prelu", "xielu"):
+        if name in hf:
+            with pytest.raises(NotImplementedError):
+                activation_kind(hf[name])
+    with pytest.raises(NotImplementedError):
+        activation_kind(torch.nn.LeakyReLU(0.2))  # only the table's slope, 0.01, has a kernel
+    with pytest.raises(NotImplementedError):
+        activation_kind(lambda x: x * x)
 
 
 def _random_params(hidden, inter, gated, post_ln, lowrank, sparse, dtype, seed, **cfg):
