@@ -203,8 +203,10 @@ int lt_dropout_mask(int64_t tokens, int32_t hidden, float p, uint64_t seed, uint
 /* C[M,N] = op(A) op(B): a_kmajor != 0: A is [M,K] row-major, else [K,M]; b_kmajor != 0: B is [N,K] row-major, else [K,N].
  * force_generic (low 4 bits): 0 the library's own choice; 1 the any-shape kernel even when a tiled bf16 kernel applies;
  * 2 the register-staged tiled kernel instead of the copy-based one.  Bits 4..7, when non-zero, choose how workgroups stagger
- * their walk over k in the copy-based kernel (15: not at all) instead of the default for the layout.  The choice travels
- * with the call (no process-wide state): lt_gemm may run concurrently with every other entry point. */
+ * their walk over k in the copy-based kernel (15: not at all) instead of the default for the layout.  Bit 8: one workgroup
+ * per tile in the copy-based kernel even when there are more tiles than compute units (by default one workgroup per compute
+ * unit then loops over its tiles; both give the same bits).  The choice travels with the call (no process-wide state): lt_gemm
+ * may run concurrently with every other entry point. */
 int lt_gemm(int32_t dtype, int64_t m, int64_t n, int64_t k, const void* a, int32_t a_kmajor, const void* b,
             int32_t b_kmajor, int32_t c_dtype, void* c, int32_t force_generic, void* stream);
 

@@ -41,7 +41,7 @@ def build(verbose: bool = False, extra_flags=(), tile_timing: bool = False) -> s
     """Compile every translation unit (in parallel) and link the shared library; returns its path.
 
     tile_timing: build the instrumented library instead (csrc/libleanffn_tile_timing.so, -DLT_TILE_TIMING: the copy-based
-    GEMM kernels record per-workgroup phase timestamps; read by lean_transformer_amd/tile_timing.py).  Never loaded by the
+    GEMM kernels record per-workgroup phase timestamps; read by tile_timing.py at the repository root).  Never loaded by the
     package itself."""
     hipcc = _hipcc()
     suffix = ".tile_timing.o" if tile_timing else ".o"

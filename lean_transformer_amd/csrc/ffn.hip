@@ -597,7 +597,8 @@ extern "C" int lt_gemm(int32_t dtype, int64_t m, int64_t n, int64_t k, const voi
   p.A[0] = operand(a, a_kmajor ? k : m, a_kmajor);
   p.B[0] = operand(b, b_kmajor ? k : n, b_kmajor);
   p.epi = epi_store_params(c, n, c_dtype, nullptr);
-  p.krot = force_generic >> 4;
+  p.krot = (force_generic >> 4) & 15;
+  p.tile_loop = (force_generic >> 8) & 1;
   force_generic &= 15;
   if (force_generic == 1) return lt_launch_gemm_generic(p, EPI_STORE, dtype, dtype, (hipStream_t)stream);
   p.variant = force_generic == 2 ? 1 : 0;  // 2: the register-staged tiled kernel instead of the copy-based one

@@ -31,12 +31,12 @@
 
 #include "lt_gemm.h"
 
-// Instrumented build (-DLT_TILE_TIMING, python -m lean_transformer_amd._build --tile-timing; never the product library):
+// Instrumented build (-DLT_TILE_TIMING, python tile_timing.py --build; never the product library):
 // thread 0 of every workgroup of the copy-based kernel records the shader clock (s_memtime) when it starts, after the
 // prologue, after 16 k-steps, after the main loop and after the epilogue, and the 100 MHz real-time counter at both ends,
 // 8 words per workgroup, into the buffer whose address the environment variable LT_TILE_TIMING_BUFFER holds; copy-based
 // launch number i of the process writes region i % 6 (4096 workgroups each), i.e. one region per GEMM of an FFN step.
-// lean_transformer_amd/tile_timing.py reads them.
+// tile_timing.py (beside bench.py) reads them.
 #ifdef LT_TILE_TIMING
 int& lt_tile_timing_launch_counter();  // one counter for the whole library (defined in gemm_mfma_bf16.hip)
 #define LT_TILE_STAMP(slot)                                                          \
@@ -130,10 +130,8 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   const bool gated = (KIND == EPI_ACT_FWD) && p.epi.gated;
 
 #ifdef LT_TILE_TIMING
-  // (the FWD / DX walks have no use for the weight-gradient walk's second activation pointer: the timing buffer rides there)
   unsigned long long* const tile_stamps =
-      ((SP == SPARSE_FWD || SP == SPARSE_DX) && p.sp.act2)
-          ? reinterpret_cast<unsigned long long*>(const_cast<void*>(p.sp.act2)) + (size_t)blockIdx.x * 8 : nullptr;
+      ((SP == SPARSE_FWD || SP == SPARSE_DX) && p.tile_stamps) ? p.tile_stamps + (size_t)blockIdx.x * 8 : nullptr;
 #endif
   LT_TILE_STAMP(0);
   LT_TILE_STAMP_REALTIME(4);
@@ -628,7 +626,7 @@ template <bool KM> struct DmaOperand {
   // wavefront sub-tile.
   __device__ __forceinline__ void setup(const GemmOperand& op, int s, int64_t row0, int64_t row_limit, int64_t pair_rows,
                                         int wave, int lane) {
-    seg = s;
+    seg = __builtin_amdgcn_readfirstlane(s);
     const int64_t ld = op.ld;
     const char* ptr = reinterpret_cast<const char*>(op.ptr);
 #pragma unroll
@@ -757,8 +755,10 @@ template <int FM, int KIND, typename TX, int tile_rows, int tile_cols, bool SCAT
 __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const GemmProblem& p, float* stage, const int64_t m0,
                                                   const int64_t n0, const int wm, const int wn, const bool gated) {
   constexpr int FN = 4, WTN = 128, WTM = FM * 32;
-  // the lane index is formed anew (two v_mbcnt) rather than kept in a register across the main loop
-  const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  // the lane index is formed anew rather than kept in a register across the main loop, through an asm statement so that a
+  // workgroup that loops over tiles does not keep what is derived from it alive from one tile's epilogue to the next's either
+  int lane;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
   // ---- epilogue.  The accumulators of a 32 x 32 block sit column-per-lane (register r = row 8 * (r / 4) + 4 * (lane / 32)
   //      + r % 4, column lane % 32).  Each wavefront transposes one 32-row strip of its sub-tile at a time through an LDS
   //      buffer of its own (32 x 128 floats = 16 KiB, the size of the smallest buffer) and reads it back row-major, 8
@@ -976,10 +976,15 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
   if constexpr (KIND == EPI_ACT_BWD) {
     if (epi.colsum) {
       // lanes l, l + 16, l + 32, l + 48 hold the same columns for different rows of the wavefront's WTM-row sub-tile
+      // (the shuffles name their source lane from this function's own lane number: the library routine forms one of its
+      // own, which the compiler would compute once and keep in a register through every main loop of a looping workgroup)
+      auto from_lane = [&](float v, int mask) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __builtin_bit_cast(int, v)));
+      };
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        colsum[e] += __shfl_xor(colsum[e], 16);
-        colsum[e] += __shfl_xor(colsum[e], 32);
+        colsum[e] += from_lane(colsum[e], 16);
+        colsum[e] += from_lane(colsum[e], 32);
       }
       // a sub-tile wholly past the last row has no partial row: the caller sizes the buffer for ceil(M / 128) of them
       if (lane < 16 && n0 + wn * WTN + lane * 8 < p.N && m0 + wm * WTM < p.M) {
@@ -1009,7 +1014,18 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
 //   position) and is read with v_readlane, so the k-loop issues no memory instruction for it.  A second k-segment (the
 //   low-rank term) is an ordinary one.
 template <bool A_KM, bool B_KM, int KIND, typename TX, bool K_TAIL, int GATHER = 0>
-__global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem, int tiles_m, int tiles_n) {
+  // A workgroup may loop over tiles.  Whatever the compiler finds to be the same in every tile -- values loaded from the problem
+  // description, the wavefront's LDS addresses, lane offsets -- it would compute once and keep in registers across the whole
+  // loop, epilogues included, and neither register file has room for that.  So the three roots of those values are laundered
+  // (an asm statement the compiler cannot see through) at the start of every tile and before every epilogue: the pointer to
+  // the problem description (the kernel's first argument, read through the constant address space so that the loads still
+  // move freely in between), the wavefront number and the lane number.  Each tile then has the register budget of a kernel
+  // that runs a single tile.
+  (void)problem;
+  typedef const __attribute__((address_space(4))) GemmProblem* KernargProblem;
+  KernargProblem pk = (KernargProblem)__builtin_amdgcn_kernarg_segment_ptr();
+#define p (*pk)
   static_assert(GATHER != 1 || (!A_KM && !B_KM && KIND == EPI_STORE && !K_TAIL), "gathered columns: weight-gradient layout");
   static_assert(GATHER != 2 || (A_KM && B_KM && !K_TAIL), "gathered k-blocks: forward layout");
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
@@ -1030,41 +1046,67 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   __shared__ __attribute__((aligned(1024))) bf16 b_s2[MN_ELEMS];
   __shared__ __attribute__((aligned(1024))) bf16 b_s3[MN_ELEMS];
 
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / WN, wn = wave % WN;
-  const bool gated = (KIND == EPI_ACT_FWD) && p.epi.gated;
+  auto fresh_lane = []() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+  };
+  int lane = fresh_lane();
+  int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  int wm = wave / WN, wn = wave % WN;
+  auto refresh = [&]() {
+    asm volatile("" : "+s"(pk), "+s"(wave));
+    lane = fresh_lane();
+    wm = wave / WN;
+    wn = wave % WN;
+  };
 #ifdef LT_TILE_TIMING
-  // (a dense problem has no use for the block-sparse walk's second activation pointer: the timing buffer rides there)
-  unsigned long long* const tile_stamps =
-      p.sp.act2 ? reinterpret_cast<unsigned long long*>(const_cast<void*>(p.sp.act2)) + (size_t)blockIdx.x * 8 : nullptr;
+  unsigned long long* tile_stamps = p.tile_stamps ? p.tile_stamps + (size_t)blockIdx.x * 8 : nullptr;  // 8 words per tile
 #endif
   LT_TILE_STAMP(0);
   LT_TILE_STAMP_REALTIME(4);
 
-  int pid = blockIdx.x;
+  // k-steps of the problem (kt_all), of this workgroup's slice of them (kt_total, from kt_begin; split-k: one k-segment only,
+  // slices of an even number of k-steps so that k-major blocks stay whole; below, k-step numbers are local to the slice) and
+  // of the first k-segment (kt_seg0).  Recomputed from the laundered problem description at every tile, like everything else.
+  int kt_all = 0, kt_begin = 0, kt_total = 0, kt_seg0 = 0;
+  bool gated = false;
+  auto k_steps = [&]() {
+    gated = (KIND == EPI_ACT_FWD) && p.epi.gated;
+    kt_all = (int)((p.K[0] + DK - 1) / DK) + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
+    kt_begin = 0;
+    kt_total = kt_all;
+    if (p.ksplit > 1) {
+      const int per = (((kt_all + p.ksplit - 1) / p.ksplit) + 1) & ~1;
+      kt_begin = min(kt_all, (int)blockIdx.y * per);
+      kt_total = min(per, kt_all - kt_begin);
+    }
+    kt_seg0 = p.nseg > 1 ? (int)((p.K[0] + DK - 1) / DK) : kt_total;
+  };
+  k_steps();
+
+  // A workgroup takes tiles blockIdx.x, blockIdx.x + gridDim.x, ... of the launch order (the host launches one workgroup per
+  // tile, or one per CU that loops: then the first copies of the next tile go out before the epilogue of the current one).
+  // Tile v of the launch order goes to XCD v % 8 either way; each XCD walks a contiguous range of tiles, GROUP_M tile-rows at a
+  // time.
   const int num_pid = tiles_m * tiles_n;
-  if ((num_pid & 7) == 0) pid = (pid & 7) * (num_pid >> 3) + (pid >> 3);
-  const int group = GROUP_M * tiles_n;
-  const int first_m = (pid / group) * GROUP_M;
-  const int gsz = min(tiles_m - first_m, GROUP_M);
-  const int tm = first_m + (pid % group) % gsz;
-  const int tn = (pid % group) / gsz;
-  const int64_t m0 = (int64_t)tm * BM;
-  const int64_t n0 = (int64_t)tn * (gated ? BN / 2 : BN);
+  int vb = blockIdx.x;
+  int tm = 0, tn = 0;
+  int64_t m0 = 0, n0 = 0;
+  auto place = [&](int v) {
+    int pid = v;
+    if ((num_pid & 7) == 0) pid = (pid & 7) * (num_pid >> 3) + (pid >> 3);
+    const int group = GROUP_M * tiles_n;
+    const int first_m = (pid / group) * GROUP_M;
+    const int gsz = min(tiles_m - first_m, GROUP_M);
+    tm = first_m + (pid % group) % gsz;
+    tn = (pid % group) / gsz;
+    m0 = (int64_t)tm * BM;
+    n0 = (int64_t)tn * (gated ? BN / 2 : BN);
+  };
+  place(vb);
 
   f32x16 acc[FM][FN];  // initialised in the prologue, after the first copies have gone out
-
-  const int kt_all = (int)((p.K[0] + DK - 1) / DK) + (p.nseg > 1 ? (int)((p.K[1] + DK - 1) / DK) : 0);
-  // split-k (one k-segment only): this workgroup walks k-steps [kt_begin, kt_begin + kt_total) of kt_all; the slices are
-  // an even number of k-steps long so that k-major blocks stay whole.  Below, k-step numbers are local to the slice.
-  int kt_begin = 0, kt_total = kt_all;
-  if (p.ksplit > 1) {
-    const int per = (((kt_all + p.ksplit - 1) / p.ksplit) + 1) & ~1;
-    kt_begin = min(kt_all, (int)blockIdx.y * per);
-    kt_total = min(per, kt_all - kt_begin);
-  }
-  const int kt_seg0 = p.nseg > 1 ? (int)((p.K[0] + DK - 1) / DK) : kt_total;
 
   // ---- buffer of k-step position I (k-step index mod 4) and copy targets, selected at compile time
   auto a_buf = [&](auto I) -> bf16* {
@@ -1084,12 +1126,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   // differs between XCDs.  Measured on the up- and down-projection shapes: +16 % and +25 % for two k-major operands,
   // nothing to gain for mn-major ones.
   int rot = 0;
-  if (!K_TAIL && GATHER == 0 && p.nseg == 1 && (kt_all & 1) == 0 && p.krot) {
-    const unsigned bx = blockIdx.x;
-    const unsigned r = (bx & 7) * (kt_all >> 3) +
-                       (p.krot == 1 ? ((bx >> 3) & 3) * (kt_all >> 5) : ((bx >> 3) & 7) * (kt_all >> 6));
-    rot = __builtin_amdgcn_readfirstlane((int)((r % (unsigned)kt_all) & ~1u));
-  }
+  auto set_rot = [&](int v) {
+    if (!K_TAIL && GATHER == 0 && p.nseg == 1 && (kt_all & 1) == 0 && p.krot) {
+      const unsigned bx = (unsigned)v;
+      const unsigned r = (bx & 7) * (kt_all >> 3) +
+                         (p.krot == 1 ? ((bx >> 3) & 3) * (kt_all >> 5) : ((bx >> 3) & 7) * (kt_all >> 6));
+      rot = __builtin_amdgcn_readfirstlane((int)((r % (unsigned)kt_all) & ~1u));
+    }
+  };
+  set_rot(vb);
   auto rotated = [&](int ks) {
     const int r = ks + rot;
     return r >= kt_all ? r - kt_all : r;
@@ -1097,17 +1142,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   DmaOperand<A_KM> ca;
   DmaOperand<B_KM> cb;
   int list_entry = 0;  // GATHER == 2: lane e holds entry e of this tile's list
-  if constexpr (GATHER == 2) {
-    const int e = min(lane, p.sp.blocks_per_out - 1);
-    const int flat = p.sp.forward_indices[(n0 / 64) * p.sp.blocks_per_out + e];
-    list_entry = (flat / p.sp.blocks_per_in) << 16 | flat;
-  }
+  auto load_list = [&]() {
+    if constexpr (GATHER == 2) {
+      const int e = min(lane, p.sp.blocks_per_out - 1);
+      const int flat = p.sp.forward_indices[(n0 / 64) * p.sp.blocks_per_out + e];
+      list_entry = (flat / p.sp.blocks_per_in) << 16 | flat;
+    }
+  };
+  load_list();
   auto setup_a = [&](int seg) {
     if (GATHER == 2 && seg == 0) {
       const GemmOperand x = {p.sp.act, p.sp.ld_act, 1};
       ca.setup(x, 0, m0, p.M, 0, wave, lane);  // unit u = column block u of X
     } else {
-      ca.setup(p.A[seg], seg, m0, p.M, 0, wave, lane);
+      const GemmOperand a = {p.A[seg].ptr, p.A[seg].ld, p.A[seg].kmajor};
+      ca.setup(a, seg, m0, p.M, 0, wave, lane);
     }
   };
   auto setup_b = [&](int seg) {
@@ -1125,9 +1174,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
         const int entry = min(tn * 4 + j, p.sp.blocks_per_out - 1);
         blocks[j] = p.sp.forward_indices[(int64_t)tm * 4 * p.sp.blocks_per_out + entry] / p.sp.blocks_per_in;
       }
-      cb.setup_gather(p.B[0], blocks, wave, lane);
+      const GemmOperand b = {p.B[0].ptr, p.B[0].ld, p.B[0].kmajor};
+      cb.setup_gather(b, blocks, wave, lane);
     } else {
-      cb.setup(p.B[seg], seg, n0, p.N, (B_KM && gated) ? p.N : 0, wave, lane);
+      const GemmOperand b = {p.B[seg].ptr, p.B[seg].ld, p.B[seg].kmajor};
+      cb.setup(b, seg, n0, p.N, (B_KM && gated) ? p.N : 0, wave, lane);
     }
   };
   setup_a(0);
@@ -1136,7 +1187,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   auto copy_a = [&](auto steady, auto I, int t, auto J0, auto J1) {
     int seg = ca.seg;
     if constexpr (!decltype(steady)::value) {  // the steady loop never crosses a k-segment boundary
-      seg = t >= kt_seg0;
+      seg = __builtin_amdgcn_readfirstlane((int)(t >= kt_seg0));  // wavefront-uniform: keep it in a scalar register
       if (seg != ca.seg) setup_a(seg);
     }
     const int ks = rotated(seg ? t - kt_seg0 : t + kt_begin);
@@ -1147,7 +1198,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   auto copy_b = [&](auto steady, auto I, int t, auto J0, auto J1) {
     int seg = cb.seg;
     if constexpr (!decltype(steady)::value) {
-      seg = t >= kt_seg0;
+      seg = __builtin_amdgcn_readfirstlane((int)(t >= kt_seg0));  // wavefront-uniform: keep it in a scalar register
       if (seg != cb.seg) setup_b(seg);
     }
     const int ks = rotated(seg ? t - kt_seg0 : t + kt_begin);
@@ -1287,87 +1338,150 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem p, int t
   using P2 = std::integral_constant<int, 2>;
   using P3 = std::integral_constant<int, 3>;
 
-  // ---- prologue: k-steps 0..2 (k-major: block 0 and the slot-0 halves of block 1) in flight and landed, first half of
-  //      k-step 0 issued
+  // ---- prologue of a tile, in two parts.  Early: k-steps 0 and 1 (k-major: block 0), into buffers the epilogue's staging
+  //      leaves alone, so that a looping workgroup issues them for its next tile before the epilogue of the current one.
+  //      Late: k-step 2 and the slot-0 halves of block 1, into the staging buffers, once the epilogue is done.  Same issue
+  //      order as the steady loop's.
+  auto prologue_early = [&]() {
+    if constexpr (A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J8{});
+    if constexpr (B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J8{});
+    if constexpr (!A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J4{});
+    if constexpr (!B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J4{});
+    if (kt_total > 1) {
+      if constexpr (!A_KM) copy_a(Ragged{}, P1{}, 1, J0{}, J4{});
+      if constexpr (!B_KM) copy_b(Ragged{}, P1{}, 1, J0{}, J4{});
+    }
+  };
+  auto prologue_late = [&]() {
+    if (kt_total > 2) {
+      if constexpr (!A_KM) copy_a(Ragged{}, P2{}, 2, J0{}, J4{});
+      if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2, J0{}, J4{});
+      if constexpr (N_KM > 0) copy_block_halves(Ragged{}, std::integral_constant<int, 0>{}, P2{}, 2);
+    }
+  };
+  constexpr int LATE_COPIES = (A_KM ? 0 : HALF) + (B_KM ? 0 : HALF) + slot_copies(0);
   LT_TILE_STAMP(6);
-  if constexpr (A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J8{});
-  if constexpr (B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J8{});
-  if constexpr (!A_KM) copy_a(Ragged{}, P0{}, 0, J0{}, J4{});
-  if constexpr (!B_KM) copy_b(Ragged{}, P0{}, 0, J0{}, J4{});
-  if (kt_total > 1) {
-    if constexpr (!A_KM) copy_a(Ragged{}, P1{}, 1, J0{}, J4{});
-    if constexpr (!B_KM) copy_b(Ragged{}, P1{}, 1, J0{}, J4{});
-  }
-  if (kt_total > 2) {
-    if constexpr (!A_KM) copy_a(Ragged{}, P2{}, 2, J0{}, J4{});
-    if constexpr (!B_KM) copy_b(Ragged{}, P2{}, 2, J0{}, J4{});
-    if constexpr (N_KM > 0) copy_block_halves(Ragged{}, std::integral_constant<int, 0>{}, P2{}, 2);
-  }
-  // The accumulators start at the bias of their column (a lane holds one column per 32-wide block), so no epilogue has to
-  // add it.  The bias loads wait behind the first copies rather than in front of them.  Gated forward: blocks 0, 1 of a
-  // wavefront are gate columns, 2, 3 the matching linear columns.
-  float bias0[FN];
-#pragma unroll
-  for (int j = 0; j < FN; j++) {
-    bias0[j] = 0.f;
-    if (p.epi.bias) {
-      // columns past N (a tile that sticks out) take the last column's bias and are never written
-      const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) +
-                                      min(n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31), p.N - 1)
-                                : min(n0 + wn * WTN + j * 32 + (lane & 31), p.N - 1);
-      bias0[j] = p.epi.bias[col];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < FM; i++)
-#pragma unroll
-    for (int j = 0; j < FN; j++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = bias0[j];
-  wait_copies_and_barrier<0>();
-  LT_TILE_STAMP(1);
-  load_frags(P0{}, 0, af[0], bfr[0]);
-  first_half(Ragged{}, P0{}, 0);
-
-  // loop body i of a group of four: second half of k-step kt + i, first half of k-step kt + i + 1
-  int kt = 0;
+  prologue_early();
   for (;;) {
-    // copies issued by the steady loop reach k-step kt + 7: they must exist and lie in the k-segment both operands' copy
-    // offsets are set up for
-    const int bound = (ca.seg == 0 && p.nseg > 1) ? kt_seg0 : kt_total;
-    if (ca.seg == cb.seg) {
-      for (; kt + 7 < bound; kt += 4) {
-#ifdef LT_TILE_TIMING
-        if (kt == 16) LT_TILE_STAMP(7);
-#endif
-        second_half(Steady{}, P0{}, kt);
-        first_half(Steady{}, P1{}, kt + 1);
-        second_half(Steady{}, P1{}, kt + 1);
-        first_half(Steady{}, P2{}, kt + 2);
-        second_half(Steady{}, P2{}, kt + 2);
-        first_half(Steady{}, P3{}, kt + 3);
-        second_half(Steady{}, P3{}, kt + 3);
-        first_half(Steady{}, P0{}, kt + 4);
+    refresh();
+    k_steps();
+    setup_a(0);
+    setup_b(0);
+    prologue_late();
+    // The accumulators start at the bias of their column (a lane holds one column per 32-wide block), so no epilogue has to
+    // add it.  The bias loads wait behind the first copies rather than in front of them.  Gated forward: blocks 0, 1 of a
+    // wavefront are gate columns, 2, 3 the matching linear columns.
+    {
+      float bias0[FN];
+#pragma unroll
+      for (int j = 0; j < FN; j++) {
+        bias0[j] = 0.f;
+        if (p.epi.bias) {
+          // columns past N (a tile that sticks out) take the last column's bias and are never written
+          const int64_t col = gated ? (j >= FN / 2 ? p.epi.inter : 0) +
+                                          min(n0 + wn * (WTN / 2) + (j % (FN / 2)) * 32 + (lane & 31), p.N - 1)
+                                    : min(n0 + wn * WTN + j * 32 + (lane & 31), p.N - 1);
+          bias0[j] = p.epi.bias[col];
+        }
       }
+#pragma unroll
+      for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][j][r] = bias0[j];
     }
-    if (kt >= kt_total) break;
-    second_half(Ragged{}, P0{}, kt);
-    if (kt + 1 < kt_total) { first_half(Ragged{}, P1{}, kt + 1); second_half(Ragged{}, P1{}, kt + 1); }
-    if (kt + 2 < kt_total) { first_half(Ragged{}, P2{}, kt + 2); second_half(Ragged{}, P2{}, kt + 2); }
-    if (kt + 3 < kt_total) { first_half(Ragged{}, P3{}, kt + 3); second_half(Ragged{}, P3{}, kt + 3); }
-    if (kt + 4 < kt_total) first_half(Ragged{}, P0{}, kt + 4);
-    kt += 4;
-    if (kt >= kt_total) break;
-  }
-  __syncthreads();  // every wavefront is done with the buffers: they become epilogue staging space
-  LT_TILE_STAMP(2);
+    // everything older than the late copies has landed (the early copies; a looping workgroup's previous stores)
+    if (kt_total > 2) wait_copies_and_barrier<LATE_COPIES>();
+    else wait_copies_and_barrier<0>();
+    LT_TILE_STAMP(1);
+    load_frags(P0{}, 0, af[0], bfr[0]);
+    first_half(Ragged{}, P0{}, 0);
 
-  // 16 KiB of staging space per wavefront: the first two buffers of each operand
-  bf16* const stage_buf = wave == 0 ? (A_KM ? a_d0 : a_s0) : wave == 1 ? (A_KM ? a_d1 : a_s1) : wave == 2 ? (B_KM ? b_d0 : b_s0) : (B_KM ? b_d1 : b_s1);
-  dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER == 1>(acc, p, reinterpret_cast<float*>(stage_buf), m0, n0, wm, wn, gated);
-  LT_TILE_STAMP(3);
-  LT_TILE_STAMP_REALTIME(5);
+    // loop body i of a group of four: second half of k-step kt + i, first half of k-step kt + i + 1
+    int kt = 0;
+    for (;;) {
+      // copies issued by the steady loop reach k-step kt + 7: they must exist and lie in the k-segment both operands' copy
+      // offsets are set up for
+      const int bound = (ca.seg == 0 && p.nseg > 1) ? kt_seg0 : kt_total;
+      if (ca.seg == cb.seg) {
+        for (; kt + 7 < bound; kt += 4) {
+#ifdef LT_TILE_TIMING
+          if (kt == 16) LT_TILE_STAMP(7);
+#endif
+          second_half(Steady{}, P0{}, kt);
+          first_half(Steady{}, P1{}, kt + 1);
+          second_half(Steady{}, P1{}, kt + 1);
+          first_half(Steady{}, P2{}, kt + 2);
+          second_half(Steady{}, P2{}, kt + 2);
+          first_half(Steady{}, P3{}, kt + 3);
+          second_half(Steady{}, P3{}, kt + 3);
+          first_half(Steady{}, P0{}, kt + 4);
+        }
+      }
+      if (kt >= kt_total) break;
+      second_half(Ragged{}, P0{}, kt);
+      if (kt + 1 < kt_total) { first_half(Ragged{}, P1{}, kt + 1); second_half(Ragged{}, P1{}, kt + 1); }
+      if (kt + 2 < kt_total) { first_half(Ragged{}, P2{}, kt + 2); second_half(Ragged{}, P2{}, kt + 2); }
+      if (kt + 3 < kt_total) { first_half(Ragged{}, P3{}, kt + 3); second_half(Ragged{}, P3{}, kt + 3); }
+      if (kt + 4 < kt_total) first_half(Ragged{}, P0{}, kt + 4);
+      kt += 4;
+      if (kt >= kt_total) break;
+    }
+    __syncthreads();  // every wavefront is done with the buffers: the early ones may take the next tile, the late ones stage
+    LT_TILE_STAMP(2);
+
+    refresh();
+    k_steps();
+    const int64_t epi_m0 = m0, epi_n0 = n0;
+    const int next = vb + (int)gridDim.x;
+    const bool more = next < num_pid;
+    if (more) {
+      place(next);
+      set_rot(next);
+      load_list();
+      setup_a(0);
+      setup_b(0);
+      prologue_early();
+    }
+    // 16 KiB of staging space per wavefront, in the buffers the early copies do not touch
+    bf16* const stage_buf = wave == 0   ? (A_KM ? a_d1 : a_s2)
+                            : wave == 1 ? (A_KM ? a_d1 + KM_ELEMS / 2 : a_s3)
+                            : wave == 2 ? (B_KM ? b_d1 : b_s2)
+                                        : (B_KM ? b_d1 + KM_ELEMS / 2 : b_s3);
+    dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER == 1>(acc, *(const GemmProblem*)pk, reinterpret_cast<float*>(stage_buf), epi_m0,
+                                                          epi_n0, wm, wn, gated);
+    LT_TILE_STAMP(3);
+    LT_TILE_STAMP_REALTIME(5);
+    if (!more) break;
+    vb = next;
+    __syncthreads();  // the staging buffers are free: the late copies may go out
+#ifdef LT_TILE_TIMING
+    if (tile_stamps) tile_stamps = p.tile_stamps + (size_t)vb * 8;
+#endif
+    LT_TILE_STAMP(0);
+    LT_TILE_STAMP_REALTIME(4);
+    LT_TILE_STAMP(6);
+  }
   static_assert(32 * WTN * 4 <= MN_ELEMS * 2, "a 32-row strip must fit the smallest buffer");
+#undef p
+}
+
+// Workgroups of a copy-based launch with `tiles` tiles: one per tile, or, when there are more tiles than compute units and
+// the problem allows it, one per compute unit that loops over tiles v, v + grid, ... (the kernel's LDS use keeps it alone on
+// its CU either way).  The looping workgroup issues the first copies of its next tile before the epilogue of the current
+// one, which takes the start of a tile (workgroup launch, first operand blocks arriving) off the critical path.
+inline unsigned dma_grid(const GemmProblem& p, int tiles) {
+  static int cus[64] = {};  // per device; filled on first use (every thread writes the same value)
+  int dev = 0;
+  if (p.tile_loop == 1 || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return (unsigned)tiles;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = -1;
+    cus[dev] = n;
+  }
+  const int n = cus[dev] & ~7;  // a multiple of the 8 XCDs, so that a workgroup's tiles stay on its XCD's range
+  return (n > 0 && tiles > n) ? (unsigned)n : (unsigned)tiles;
 }
 
 template <bool A_KM, bool B_KM, int KIND>
@@ -1375,7 +1489,7 @@ int launch_dma(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
   GemmProblem p = problem;
 #ifdef LT_TILE_TIMING
   if (const char* e = getenv("LT_TILE_TIMING_BUFFER"))
-    p.sp.act2 = (const void*)(strtoull(e, nullptr, 0) + (size_t)(lt_tile_timing_launch_counter()++ % 6) * 4096 * 64);
+    p.tile_stamps = (unsigned long long*)(strtoull(e, nullptr, 0) + (size_t)(lt_tile_timing_launch_counter()++ % 6) * 4096 * 64);
 #endif
   // k-walk stagger: on unless the caller chose (15: off)
   if (p.krot == 0) p.krot = (A_KM && B_KM) ? 2 : 0;
@@ -1385,7 +1499,7 @@ int launch_dma(const GemmProblem& problem, int io_dtype, hipStream_t stream) {
   const int tiles_n = (int)((p.N + (gated ? 127 : 255)) / (gated ? 128 : 256));
   bool k_tail = false;
   for (int s = 0; s < p.nseg; s++) k_tail = k_tail || (p.K[s] % DK != 0);
-  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(p.ksplit > 1 ? p.ksplit : 1)), block(256);
+  dim3 grid(dma_grid(p, tiles_m * tiles_n), (unsigned)(p.ksplit > 1 ? p.ksplit : 1)), block(256);
   const bool bf16_io = KIND == EPI_OUT && io_dtype == LT_BF16;
   if constexpr (!A_KM && !B_KM) {
     if (k_tail) {
@@ -1432,7 +1546,7 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
   // block-sparse FWD / DX launch number i of the process writes region i % 4 (8192 workgroups each) of its own buffer
   if (const char* e = getenv("LT_TILE_TIMING_BUFFER_SPARSE")) {
     if (p.sp.mode == SPARSE_FWD || p.sp.mode == SPARSE_DX)
-      p.sp.act2 = (const void*)(strtoull(e, nullptr, 0) + (size_t)(lt_tile_timing_launch_counter()++ % 4) * 8192 * 64);
+      p.tile_stamps = (unsigned long long*)(strtoull(e, nullptr, 0) + (size_t)(lt_tile_timing_launch_counter()++ % 4) * 8192 * 64);
   }
 #endif
   const SparseWalk& sp = p.sp;
@@ -1447,10 +1561,9 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
         // runs of 4 output blocks share one list: a dense product over gathered k-blocks on 256 x 256 tiles
         GemmProblem q = p;
         q.K[0] = (int64_t)sp.blocks_per_out * 64;
-        q.sp.act2 = nullptr;
         q.ksplit = 0; q.krot = 0;
         const int tiles_n = (int)(p.N / 256);
-        hipLaunchKernelGGL((gemm_bf16_dma_kernel<true, true, KIND, float, false, 2>), dim3((unsigned)(tiles_m * tiles_n)), block, 0,
+        hipLaunchKernelGGL((gemm_bf16_dma_kernel<true, true, KIND, float, false, 2>), dim3(dma_grid(q, tiles_m * tiles_n)), block, 0,
                            stream, q, tiles_m, tiles_n);
         LT_LAUNCH_CHECK();
         return LT_OK;
@@ -1480,9 +1593,8 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
         q.nseg = 1; q.K[0] = sp.tokens; q.K[1] = 0;
         q.A[0].ptr = sp.act; q.A[0].ld = sp.ld_act; q.A[0].kmajor = 0;
         q.B[0].ptr = sp.act2; q.B[0].ld = sp.ld_act2; q.B[0].kmajor = 0;
-        q.sp.act2 = nullptr;
         q.ksplit = 0; q.krot = 0;
-        hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, 1>), dim3((unsigned)(tiles_m * tiles_n)),
+        hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, 1>), dim3(dma_grid(q, tiles_m * tiles_n)),
                            block, 0, stream, q, tiles_m, tiles_n);
         LT_LAUNCH_CHECK();
         return LT_OK;

@@ -83,6 +83,9 @@ struct GemmProblem {
   int64_t split_stride;
   int krot;  // copy-based kernel: how workgroups stagger their walk over k (0: all start at k = 0)
   int variant;  // tiled bf16 kernels: 0 the launcher's choice, 1 the register-staged kernel where the copy-based one applies
+  int tile_loop;  // copy-based kernel: 0 the launcher's choice (one workgroup per CU that loops over its tiles when there are
+                  // more tiles than CUs), 1 one workgroup per tile
+  unsigned long long* tile_stamps;  // instrumented build only (-DLT_TILE_TIMING): 8 words of clock stamps per tile; else null
 };
 
 // ---------------------------------------------------------------------------------------------------------------------

@@ -57,7 +57,7 @@ def act_forward(kind: str, x: torch.Tensor) -> torch.Tensor:
     if kind == "gelu_10":
         return torch.clip(F.gelu(x), -10, 10)
     if kind == "relu6":
-        return torch.clamp(x, 0, 6)
+        return F.relu6(x)  # (autograd of relu6 is 0 at both kinks; of clamp(x, 0, 6) it would be 1)
     if kind == "relu2":
         return torch.square(F.relu(x))
     if kind == "leaky_relu":

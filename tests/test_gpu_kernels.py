@@ -90,6 +90,33 @@ def _kernel_tags(fn):
     return out, tags
 
 
+TILE_LOOP_CASES = [(a, b, m, n, k) for a, b in ((True, True), (True, False), (False, False))
+                   for m, n, k in ((4352, 4096, 192), (4360, 4104, 320), (8192, 8192, 64))] + [(False, False, 4352, 4096, 200)]
+
+
+@pytest.mark.parametrize("a_kmajor,b_kmajor,m,n,k", TILE_LOOP_CASES)
+def test_gemm_tile_loop_gives_the_same_bits_as_one_workgroup_per_tile(a_kmajor, b_kmajor, m, n, k):
+    """more tiles than compute units: by default one workgroup per compute unit loops over its tiles and issues the first
+    copies of its next tile before the epilogue of the current one; flag bit 8 launches one workgroup per tile instead.
+    Same arithmetic in the same order: the results must be identical, whole tiles, tiles past the edge and a ragged
+    reduction (mn-major operands) alike, and right."""
+    g = torch.Generator(device=DEV).manual_seed(m + n + k)
+    a = torch.randn((m, k) if a_kmajor else (k, m), generator=g, device=DEV).to(torch.bfloat16)
+    b = torch.randn((n, k) if b_kmajor else (k, n), generator=g, device=DEV).to(torch.bfloat16)
+    ref = (a.float() if a_kmajor else a.float().t()) @ (b.float().t() if b_kmajor else b.float())
+    for c_dtype in (torch.float32, torch.bfloat16):
+        flat = torch.full((2, m * n + 4096), 7.0, dtype=c_dtype, device=DEV)  # two results, each with a guard behind it
+        for i, force in enumerate((0, 1 << 8)):
+            c = flat[i, :m * n].view(m, n)
+            _, tags = _kernel_tags(lambda: nat.check(
+                nat.lib().lt_gemm(nat.dtype_code(a.dtype), m, n, k, nat.ptr(a), int(a_kmajor), nat.ptr(b), int(b_kmajor),
+                                  nat.dtype_code(c_dtype), nat.ptr(c), force, nat.current_stream(c.device)), "lt_gemm"))
+            assert any(t.startswith("gemm_bf16_") and t.endswith("_store") for t in tags), tags
+        assert torch.equal(flat[0], flat[1])
+        assert bool((flat[:, m * n:] == 7.0).all())
+        assert rel_err(flat[0, :m * n].view(m, n).float(), ref) <= (1e-5 if c_dtype == torch.float32 else 1e-2)
+
+
 @pytest.mark.parametrize("a_kmajor,b_kmajor,tag", [(True, True, "gemm_bf16_nt_store"), (True, False, "gemm_bf16_nn_store"),
                                                    (False, False, "gemm_bf16_tn_store")])
 @pytest.mark.parametrize("m,n,k", [(512, 320, 128), (256, 8, 64), (328, 200, 192), (1600, 1608, 320), (264, 776, 448)])

@@ -1,8 +1,7 @@
 """Where the cycles of each GEMM launch of a LeanFFN step go: prologue, main loop, epilogue, per workgroup (= per tile).
 
-    python -m lean_transformer_amd._build --tile-timing      (once: builds csrc/libleanffn_tile_timing.so)
-    python -m lean_transformer_amd.tile_timing --config c3    (on the GPU; c2: the other dense configuration; c4: the
-                                                               block-sparse one)
+    python tile_timing.py --build          (once, no GPU needed: builds lean_transformer_amd/csrc/libleanffn_tile_timing.so)
+    python tile_timing.py --config c3      (on the GPU; c2: the other dense configuration; c4: the block-sparse one)
 
 Runs fwd+bwd steps of a benchmark configuration (bench.py's) on the instrumented library, in which thread 0 of every
 workgroup of the copy-based GEMM kernel stamps the shader clock (s_memtime) at its phase boundaries and the 100 MHz
@@ -11,7 +10,8 @@ into prologue (launch to first matrix instruction), main loop (with the first 16
 (1 024 ticks per 32-wide k-step: 32 matrix instructions of 32 cycles per SIMD) and the shader clock while tiles run.
 With --config c4 the stamped kernels are the block-sparse forward / input-gradient walks (256 x 64 tiles, two workgroups per
 CU): start, before the first operand loads, after the main loop, after the epilogue.
-A measurement tool: nothing in the package imports it.
+A measurement tool beside bench.py, whose workloads it runs: not part of the package, and the package never loads the
+instrumented library.
 """
 import argparse
 import os
@@ -22,15 +22,21 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4"], help="bf16 benchmark configuration of bench.py")
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--build", action="store_true", help="compile the instrumented library (hipcc, no GPU needed) and exit")
     args = ap.parse_args()
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    root = os.path.dirname(os.path.abspath(__file__))
     sys.path.insert(0, root)
+    from lean_transformer_amd import _build
+
+    if args.build:
+        print(_build.build(tile_timing=True))
+        return
     import torch
 
-    from lean_transformer_amd import _build, _native as nat
+    from lean_transformer_amd import _native as nat
 
     if not os.path.exists(_build.TILE_TIMING_LIB_PATH):
-        sys.exit(f"{_build.TILE_TIMING_LIB_PATH} is missing: run `python -m lean_transformer_amd._build --tile-timing`")
+        sys.exit(f"{_build.TILE_TIMING_LIB_PATH} is missing: run `python tile_timing.py --build`")
     nat.LIB_PATH = _build.TILE_TIMING_LIB_PATH  # before the first nat.lib() call
     import bench
     import lean_transformer_amd as lt
