@@ -81,7 +81,9 @@ typedef struct lt_linear {
                              blocks, and under each of them the run's weight blocks are adjacent (forward_indices of output
                              block ob0 + j = those of ob0, + j).  PixelFly with stretch=True on a tall matrix: out_blocks /
                              in_blocks.  A promise by the caller that only selects faster forward and weight-gradient
-                             kernels; 0 or 1 when not known. */
+                             kernels; 0 or 1 when not known, which is always safe.  Must divide the number of output blocks.
+                             A false promise computes with the wrong weight blocks (it cannot make a kernel read outside
+                             the weight); lt_linear_check_out_group tests it on the device. */
   int32_t reserved;       /* 0 */
 } lt_linear;
 
@@ -158,6 +160,12 @@ int lt_linear_backward(const lt_linear* lin, int64_t tokens, int32_t dtype, cons
                        const void* lowrank_hid, void* dx, const lt_linear_grads* grads, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* Tests lin->out_group against lin->forward_indices on the device: writes 1 to *flag (device memory, 4 bytes) when every
+ * aligned run of out_group output blocks shares one list of input blocks with adjacent weight blocks, else 0.  Asynchronous
+ * like everything else: the caller reads the flag when it chooses (once per index table is enough).  No counterpart in the
+ * reference, whose matmul takes no such hint. */
+int lt_linear_check_out_group(const lt_linear* lin, int32_t* flag, void* stream);
+
 /* ---- block-sparse matmul alone (weight in the native [in_features, A, block] format) ----------------------------------- */
 int lt_blocksparse_forward(const lt_linear* lin, int64_t tokens, int32_t dtype, const void* x, void* y, void* stream);
 /* dx and/or dweight may be NULL */
@@ -182,7 +190,10 @@ int lt_layernorm_backward(int64_t tokens, int32_t hidden, int32_t x_dtype, const
  * looked up on the first call on each device.  The device that owns `stream` must be the current device.  Rows of a
  * multiple of 4 elements with 16-byte aligned pointers fit for every tokens / hidden <= 8192; other shapes are refused
  * with LT_ERR_UNSUPPORTED once tokens * hidden * 8 bytes (tokens capped at 1024) exceed the buffer.  Calls no allocator.
- * All calls on one GPU share the buffer: calls that overlap in time on the same GPU (different streams) race. */
+ * All calls on one GPU share the buffer: calls that overlap in time on the same GPU (different streams, or two captured
+ * graphs replayed side by side) race.  The buffer's address is looked up on the first call on each device, which must
+ * therefore happen outside stream capture (one warm-up call per device): a first call on a capturing stream is refused with
+ * LT_ERR_UNSUPPORTED and leaves the capture intact. */
 size_t lt_layernorm_backward_static_scratch_bytes(void);
 int lt_layernorm_backward_static(int64_t tokens, int32_t hidden, int32_t x_dtype, const void* x, const float* stats,
                                  const float* weight, int32_t dy_dtype, const void* dy, int32_t dx_dtype,

@@ -20,7 +20,7 @@ _DTYPES = {torch.float32: LT_F32, torch.bfloat16: LT_BF16}
 EXPORTED_SYMBOLS = (
     "lt_version", "lt_last_error",
     "lt_ffn_forward_workspace_bytes", "lt_ffn_backward_workspace_bytes", "lt_ffn_forward", "lt_ffn_backward",
-    "lt_linear_backward_workspace_bytes", "lt_linear_forward", "lt_linear_backward",
+    "lt_linear_backward_workspace_bytes", "lt_linear_forward", "lt_linear_backward", "lt_linear_check_out_group",
     "lt_blocksparse_forward", "lt_blocksparse_backward",
     "lt_layernorm_forward", "lt_layernorm_backward_workspace_bytes", "lt_layernorm_backward",
     "lt_layernorm_backward_static_scratch_bytes", "lt_layernorm_backward_static",
@@ -83,6 +83,7 @@ def _declare(lib):
     lib.lt_linear_backward_workspace_bytes.restype = c_size_t
     lib.lt_linear_backward_workspace_bytes.argtypes = [POINTER(LtLinear), c_int64, c_int32]
     lib.lt_linear_forward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.lt_linear_check_out_group.argtypes = [POINTER(LtLinear), c_void_p, c_void_p]
     lib.lt_linear_backward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                        POINTER(LtLinearGrads), c_void_p, c_size_t, c_void_p]
     lib.lt_blocksparse_forward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p]
@@ -111,6 +112,12 @@ def _declare(lib):
         fn = getattr(lib, name)
         if fn.restype is ctypes.c_int:  # default restype: these return lt_status
             fn.restype = c_int32
+
+
+def available() -> bool:
+    """whether the built library is there (the only caller: the stock-op path's choice of dropout mask; every kernel path
+    calls lib() and fails loudly without it)"""
+    return _lib is not None or os.path.exists(LIB_PATH)
 
 
 def lib():

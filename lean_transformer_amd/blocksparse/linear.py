@@ -164,8 +164,12 @@ def shared_list_run(forward_indices: torch.Tensor, blocks_per_in: int) -> int:
     return run
 
 
-def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices, backward_indices) -> "nat.LtLinear":
-    """ctypes descriptor of one projection; all tensors already in their final dtype and contiguous"""
+def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices, backward_indices,
+                index_owner: Optional[torch.Tensor] = None) -> "nat.LtLinear":
+    """ctypes descriptor of one projection; all tensors already in their final dtype and contiguous.  index_owner: the
+    caller's own forward_indices tensor (the module's buffer) when `forward_indices` may be a converted copy of it: the
+    shared-list run is remembered on that object, so that a copy made per call does not recompute it (and synchronise) per
+    call."""
     desc = nat.LtLinear()
     desc.weight = nat.ptr(weight)
     desc.bias = nat.ptr(bias_f32)
@@ -179,7 +183,10 @@ def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices
         desc.in_features, desc.out_features = in_features, forward_indices.shape[0] * block
         desc.block, desc.blocks_per_in, desc.blocks_per_out = block, blocks_per_in, forward_indices.shape[1]
         desc.forward_indices, desc.backward_indices = nat.ptr(forward_indices), nat.ptr(backward_indices)
-        desc.out_group = shared_list_run(forward_indices, blocks_per_in) if forward_indices is not None else 0
+        owner = forward_indices if index_owner is None else index_owner
+        desc.out_group = shared_list_run(owner, blocks_per_in)
+        if desc.out_group > 1 and forward_indices.shape[0] % desc.out_group:
+            desc.out_group = 1  # (cannot happen for a power of two that divides the block count; the C ABI refuses it)
     return desc
 
 
@@ -203,7 +210,7 @@ class _GeneralizedLinear(torch.autograd.Function):
         b32 = _as(bias, torch.float32)
         fwd = None if forward_indices is None else forward_indices.to(torch.int32).contiguous()
         bwd = None if backward_indices is None else backward_indices.to(torch.int64).contiguous()
-        desc = linear_desc(w, b32, l1, l2, fwd, bwd)
+        desc = linear_desc(w, b32, l1, l2, fwd, bwd, forward_indices)
         if x.shape[1] != desc.in_features:
             raise ValueError(f"input has {x.shape[1]} features, the weight takes {desc.in_features}")
         tokens = x.shape[0]
@@ -228,7 +235,7 @@ class _GeneralizedLinear(torch.autograd.Function):
         l1, l2 = _as(lowrank_first, dtype), _as(lowrank_second, dtype)
         fwd = None if forward_indices is None else forward_indices.to(torch.int32).contiguous()
         bwd = None if backward_indices is None else backward_indices.to(torch.int64).contiguous()
-        desc = linear_desc(w, None, l1, l2, fwd, bwd)
+        desc = linear_desc(w, None, l1, l2, fwd, bwd, forward_indices)
         tokens = x.shape[0]
         grads = nat.LtLinearGrads()
         dx = torch.empty_like(x) if need[0] else None

@@ -24,13 +24,13 @@ def _sparse_desc(weight: torch.Tensor, forward_indices: Optional[torch.Tensor], 
 
 
 def blocksparse_matmul(input: torch.Tensor, weight: torch.Tensor, forward_indices: torch.Tensor) -> torch.Tensor:
-    """
-    :param input: tensor [*batch_dims, in_features]
-    :param weight: tensor [in_features, active_blocks_per_input, block_size]
-    :param forward_indices: the first output of get_indices_from_layout(...), int32 [num_output_blocks, K]
-    :returns: tensor [*batch_dims, out_features]
-    """
-    assert input.shape[-1] == weight.shape[0]
+    """input [..., in_features] times a block-sparse weight -> [..., out_features].
+
+    weight: the active blocks in the native order [in_features, blocks per input block, block]; forward_indices: the int32
+    table [output blocks, K] that get_indices_from_layout returns first (entry = input block * blocks per input block +
+    position of the weight block under that input block).  out_features = output blocks * block."""
+    if input.shape[-1] != weight.shape[0]:
+        raise AssertionError(f"input has {input.shape[-1]} features, the weight takes {weight.shape[0]}")
     device = nat.require_gpu(input, weight, forward_indices)
     block = weight.shape[2]
     out_features = forward_indices.shape[0] * block
@@ -51,7 +51,8 @@ def blocksparse_matmul_backward(grad_output: torch.Tensor, input: torch.Tensor, 
                                 backward_indices: torch.Tensor, input_requires_grad: bool = True,
                                 weight_requires_grad: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
     """Gradients of blocksparse_matmul w.r.t. input and/or weight; a gradient that is not requested comes back empty."""
-    assert input_requires_grad or weight_requires_grad, "computing backward but none of the inputs requires grad"
+    if not (input_requires_grad or weight_requires_grad):
+        raise AssertionError("backward was asked for neither the input's nor the weight's gradient")
     device = nat.require_gpu(grad_output, input, weight, backward_indices)
     x = input.reshape(-1, input.shape[-1]).contiguous()
     dy = grad_output.reshape(x.shape[0], -1).contiguous()

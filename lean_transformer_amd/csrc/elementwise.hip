@@ -748,6 +748,11 @@ int static_scratch_for(hipStream_t stream, void** out) {
   LT_REQUIRE(current >= 0 && current < LT_MAX_DEVICES, LT_ERR_UNSUPPORTED, "device index %d above %d", current, LT_MAX_DEVICES - 1);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[current]) {
+    // the look-up is not a stream operation: under capture it could invalidate the caller's capture, so it is refused there
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    LT_HIP(hipStreamIsCapturing(stream, &capture));
+    LT_REQUIRE(capture == hipStreamCaptureStatusNone, LT_ERR_UNSUPPORTED,
+               "layernorm backward (static scratch): the first call on a device must happen outside stream capture");
     void* ptr = nullptr;
     LT_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     LT_REQUIRE(ptr != nullptr, LT_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch");

@@ -64,6 +64,37 @@ int check_linear(const lt_linear& lin, const char* name, int tables = NEED_FWD_T
                    (int64_t)lin.blocks_per_in * (lin.in_features / lin.block) ==
                        (int64_t)lin.blocks_per_out * (lin.out_features / lin.block),
                LT_ERR_BAD_ARG, "%s: unbalanced layout (K=%d, A=%d)", name, lin.blocks_per_out, lin.blocks_per_in);
+    LT_REQUIRE(lin.out_group >= 0 && (lin.out_group <= 1 || (lin.out_features / lin.block) % lin.out_group == 0), LT_ERR_BAD_ARG,
+               "%s: out_group=%d does not divide the %d output blocks", name, lin.out_group, lin.out_features / lin.block);
+  }
+  return LT_OK;
+}
+
+namespace {
+// flag[0] = 0 when output block ob's list differs from that of the first block of its aligned run of `group`, or its weight
+// blocks do not follow that block's by ob % group (what lt_linear::out_group promises); untouched otherwise
+__global__ void check_out_group_kernel(const int32_t* __restrict__ forward_indices, int out_blocks, int per_out, int per_in,
+                                       int group, int32_t* flag) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= out_blocks * per_out) return;
+  const int ob = i / per_out, e = i % per_out, ob0 = ob - ob % group;
+  const int mine = forward_indices[i], first = forward_indices[ob0 * per_out + e];
+  if (mine / per_in != first / per_in || mine != first + (ob - ob0)) flag[0] = 0;
+}
+__global__ void set_flag_kernel(int32_t* flag, int32_t value) { flag[0] = value; }
+}  // namespace
+
+extern "C" int lt_linear_check_out_group(const lt_linear* lin, int32_t* flag, void* stream_) {
+  LT_REQUIRE(lin && flag, LT_ERR_BAD_ARG, "check out_group: null argument");
+  LT_TRY(check_linear(*lin, "check out_group", NEED_FWD_TABLE));
+  hipStream_t stream = (hipStream_t)stream_;
+  hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, stream, flag, 1);
+  LT_LAUNCH_CHECK();
+  if (lin->block > 0 && lin->out_group > 1) {
+    const int out_blocks = lin->out_features / lin->block, entries = out_blocks * lin->blocks_per_out;
+    hipLaunchKernelGGL(check_out_group_kernel, dim3((unsigned)((entries + 255) / 256)), dim3(256), 0, stream,
+                       lin->forward_indices, out_blocks, lin->blocks_per_out, lin->blocks_per_in, lin->out_group, flag);
+    LT_LAUNCH_CHECK();
   }
   return LT_OK;
 }

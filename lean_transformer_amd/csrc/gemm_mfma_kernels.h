@@ -1145,7 +1145,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
   auto load_list = [&]() {
     if constexpr (GATHER == 2) {
       const int e = min(lane, p.sp.blocks_per_out - 1);
-      const int flat = p.sp.forward_indices[(n0 / 64) * p.sp.blocks_per_out + e];
+      // (clamped so that the four blocks read from `flat` on lie inside the weight even if the caller's promise of shared
+      // lists is false: wrong results then, but no access outside the weight)
+      const int flat = min(p.sp.forward_indices[(n0 / 64) * p.sp.blocks_per_out + e],
+                           (int)(p.sp.ld_act / 64) * p.sp.blocks_per_in - 4);
       list_entry = (flat / p.sp.blocks_per_in) << 16 | flat;
     }
   };

@@ -90,10 +90,12 @@ class LeanFFN(nn.Module):
         if self.post_layer_norm is not None:
             out = self.post_layer_norm(out)
         if self.training and self.dropout:
-            if out.is_cuda:
+            if float(self.dropout) >= 1.0:
+                out = torch.zeros_like(out)  # what torch.dropout returns for p = 1 (no 1 / (1 - p) to form)
+            elif out.is_cuda and nat.available():
                 keep = philox_keep_mask(out.shape[0], width, float(self.dropout), out.device)
                 out = out * (keep.to(out.dtype) * (1.0 / (1.0 - float(self.dropout))))
-            else:
+            else:  # CPU tensors, or no built library: the stock op, as at lean_transformer/ffn.py:80
                 out = torch.dropout(out, self.dropout, True)
         if self.residual:
             out = out + rows
@@ -244,7 +246,7 @@ class _LeanFFN(torch.autograd.Function):
                        None if fwd is None else fwd.to(torch.int32).contiguous(),
                        None if bwd is None else bwd.to(torch.int64).contiguous())
             keep.append(tensors)
-            projections.append(linear_desc(*tensors))
+            projections.append(linear_desc(*tensors, index_owner=fwd))
         desc = nat.LtFfnDesc()
         desc.tokens, desc.hidden = tokens, hidden
         desc.intermediate = projections[1].in_features

@@ -55,3 +55,32 @@ def assert_close(got, ref, dtype, name=""):
     else:
         cos = cosine(got, ref)
         assert err <= BF16_TOL and cos >= BF16_COS, f"{name}: max relative error {err:.3e}, cosine {cos:.6f}"
+
+
+def assert_within_bf16_noise(named_got, named_truth, stock_runs, label="", depth=1):
+    """Deep bf16 computations (a module applied several times in a row, a whole model): rounding noise compounds, so two
+    equally valid bf16 runs differ from the fp32 truth -- and from each other -- by more than the single-application bar.
+    `named_got` / `named_truth`: {name: tensor}; `stock_runs`: two or more {name: tensor} results of stock-op bf16 runs of the
+    same computation; `depth`: how many applications of the block follow one another.  A tensor passes when it meets the bar
+    of one application (max relative error 2e-2, cosine 0.9999) scaled to `depth` independent applications -- errors add in
+    quadrature, so 2e-2 sqrt(depth), and 1 - cosine, which goes with the square of the error, 1e-4 depth -- or when both
+    figures are within 1.1 x swing x the largest of the stock-op runs' figures, swing being the largest factor by which that
+    figure moves on any tensor between two stock-op runs (measured here, per figure)."""
+    assert len(stock_runs) >= 2
+    figures = {name: [(rel_err(run[name], truth), 1.0 - cosine(run[name], truth)) for run in stock_runs]
+               for name, truth in named_truth.items()}
+    swing_err = max(max(e for e, _ in f) / max(min(e for e, _ in f), 1e-12) for f in figures.values())
+    swing_ang = max(max(a for _, a in f) / max(min(a for _, a in f), 1e-12) for f in figures.values())
+    failures = []
+    for name, truth in named_truth.items():
+        got = named_got[name]
+        assert got.shape == truth.shape and torch.isfinite(got.float()).all(), name
+        err, ang = rel_err(got, truth), 1.0 - cosine(got, truth)
+        if err <= BF16_TOL * depth ** 0.5 and ang <= (1.0 - BF16_COS) * depth:
+            continue
+        e_max, a_max = max(e for e, _ in figures[name]), max(a for _, a in figures[name])
+        if err > 1.1 * swing_err * e_max or ang > 1.1 * swing_ang * a_max:
+            failures.append(f"{name}: max relative error {err:.3e} (stock-op bf16 runs " + " ".join(f"{e:.3e}" for e, _ in figures[name])
+                            + f", swing {swing_err:.2f}), 1 - cosine {ang:.3e} (" + " ".join(f"{a:.3e}" for _, a in figures[name])
+                            + f", swing {swing_ang:.2f})")
+    assert not failures, label + "\n" + "\n".join(failures)

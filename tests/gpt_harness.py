@@ -104,11 +104,22 @@ class OracleFFN(nn.Module):
     def __init__(self, hidden: int, intermediate: int, gated: bool, eps: float):
         super().__init__()
         self.gated, self.eps = gated, eps
+        self.lean = False  # True: the memory-lean autograd.Function of the oracle instead of the plain composition
         self.pre_layer_norm = nn.LayerNorm(hidden, eps=eps)
         self.i2h_proj = nn.Linear(hidden, intermediate * (2 if gated else 1))
         self.h2o_proj = nn.Linear(intermediate, hidden)
 
     def forward(self, x):
+        if self.lean:
+            # the reference's own schedule in stock ops (the oracle's LeanFFNFunction: saves x and the pre-activation,
+            # closed-form backward, custom_fwd / custom_bwd like _LeanFFN, so under autocast every matmul of forward and
+            # backward takes bf16 operands): a second stock-op implementation whose roundings fall elsewhere
+            p = offn.FFNParams(
+                self.pre_layer_norm.weight, self.pre_layer_norm.bias,
+                offn.LinearParams(self.i2h_proj.weight, self.i2h_proj.bias, out_features=self.i2h_proj.out_features),
+                offn.LinearParams(self.h2o_proj.weight, self.h2o_proj.bias, out_features=self.h2o_proj.out_features),
+                None, None, offn.FFNConfig(gated=self.gated, act="gelu_fused", ln_eps=self.eps, residual=True, dropout=0.0))
+            return offn.lean_ffn(x, p)
         autocast = torch.is_autocast_enabled(x.device.type)
         cast = (lambda t: t.to(torch.get_autocast_dtype(x.device.type))) if autocast else (lambda t: t)
         # under autocast the oracle follows the reference's roundings: LayerNorm in fp32, GEMM operands in bf16

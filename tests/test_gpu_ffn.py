@@ -9,7 +9,7 @@ import torch
 import torch.nn as nn
 
 import lean_transformer_amd as lt
-from conftest import assert_close
+from conftest import assert_close, assert_within_bf16_noise
 from helpers import dropout_mask, generator_position, module_tensors, oracle_params, run_oracle
 from lean_transformer_amd.utils import ACT2FN
 from oracle import ffn as offn
@@ -100,9 +100,13 @@ def test_ffn_generalized_projections(adapter_dim, lowrank_dim, block_size, resid
         assert_close(grad, ref[name], torch.float32, name)
 
 
-def _oracle_named_grads(ffn, x, dy):
-    """gradients per named module parameter, from the CPU oracle with the low-rank factors concatenated from leaves"""
-    leaves = {n: t.detach().cpu().float().clone().requires_grad_(True) for n, t in ffn.named_parameters()}
+def _oracle_with_named_leaves(ffn, shared=None, bf16_rounding=False, device="cpu"):
+    """(FFNParams, {name: leaf}) of the CPU oracle with one fp32 leaf per named module parameter: the combined low-rank
+    factors are concatenated from the shared part and the adapter.  `shared` maps names to leaves that already exist (layers
+    that share a GeneralizedMatrix share its leaves, so that autograd sums their gradients)."""
+    shared = {} if shared is None else shared
+    leaves = {n: shared[n] if n in shared else t.detach().to(device).float().clone().requires_grad_(True)
+              for n, t in ffn.named_parameters()}
 
     def proj(prefix, module):
         w = leaves[f"{prefix}.matrix.weight"]
@@ -116,11 +120,131 @@ def _oracle_named_grads(ffn, x, dy):
     p = offn.FFNParams(leaves["pre_layer_norm.weight"], leaves["pre_layer_norm.bias"], proj("i2h_proj", ffn.i2h_proj),
                        proj("h2o_proj", ffn.h2o_proj), leaves.get("post_layer_norm.weight"),
                        leaves.get("post_layer_norm.bias"),
-                       offn.FFNConfig(gated=ffn.gated, ln_eps=ffn.pre_layer_norm.eps, residual=ffn.residual))
+                       offn.FFNConfig(gated=ffn.gated, ln_eps=ffn.pre_layer_norm.eps, residual=ffn.residual,
+                                      bf16_rounding=bf16_rounding))
+    return p, leaves
+
+
+def _oracle_named_grads(ffn, x, dy):
+    """gradients per named module parameter, from the CPU oracle with the low-rank factors concatenated from leaves"""
+    p, leaves = _oracle_with_named_leaves(ffn)
     y = offn.plain_ffn(x, p)
     names = list(leaves)
     grads = torch.autograd.grad(y, [leaves[n] for n in names], dy)
     return dict(zip(names, grads))
+
+
+def _stack_objective(out):
+    """the reference's scalar objective of its stacked tests (tests/test_ffn.py:60, 219)"""
+    return (out * (out + 1)).square().mean()
+
+
+@pytest.mark.parametrize("adapter_dim,lowrank_dim,residual", [
+    (0, 0, True), (0, 0, False), (4, 0, True), (0, 4, True), (2, 6, False), (6, 2, True), (2, 2, True), (1, 1, False)])
+@pytest.mark.parametrize("custom_grad", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ffn_shared_applied_four_times(adapter_dim, lowrank_dim, residual, custom_grad, dtype):
+    """reference tests/test_ffn.py:150-241 as the reference runs it: ONE module -- PixelFly(16) projections with a shared
+    low-rank term and an adapter, gated, post-LayerNorm -- applied four times in a row, so that every parameter gradient is
+    the sum over four uses, objective (out (out + 1))^2 .mean(), with the memory-lean autograd.Function
+    (ffn_custom_grad=True) and with the stock-op composition over the HIP generalized-linear layers (False).  The reference's
+    rows: it fixes block_size = 16 inside the test, so its nine rows are these eight distinct ones.  Ground truth: autograd
+    of the CPU oracle's plain composition applied four times with one leaf per module parameter.  bf16: fp32 parameters and
+    residual stream under bf16 autocast (how the reference runs in bf16); a tensor that misses the bar of one application
+    scaled to four (4e-2, cosine 0.9996) against the fp32 truth must be within the noise of two stock-op bf16 runs of the
+    same stack (conftest: assert_within_bf16_noise)."""
+    torch.manual_seed(adapter_dim * 100 + lowrank_dim * 10 + int(residual))
+    dim, layout = 32, "pixelfly(16)"
+    ffn = lt.LeanFFN(
+        dim, 4 * dim, gated=True, post_layer_norm=True, layer_norm_eps=1e-5,
+        i2h_proj=lt.GeneralizedLinear(lt.GeneralizedMatrix(dim, 8 * dim, layout, lowrank_dim), adapter_dim),
+        h2o_proj=lt.GeneralizedLinear(lt.GeneralizedMatrix(4 * dim, dim, layout, lowrank_dim), adapter_dim),
+        residual=residual, ffn_custom_grad=custom_grad)
+    with torch.no_grad():
+        ffn.post_layer_norm.bias.normal_()
+        ffn.post_layer_norm.weight.uniform_(0.5, 1.5)
+        for proj in (ffn.i2h_proj, ffn.h2o_proj):
+            if proj.adapter_second is not None:
+                proj.adapter_second.normal_(std=0.1)  # (zero-initialised adapters would leave adapter_first without gradient)
+    ffn = ffn.to(DEV)
+    bf16 = dtype == torch.bfloat16
+    p, leaves = _oracle_with_named_leaves(ffn)
+    names = list(leaves)
+    x = torch.rand(4, 128, dim)
+
+    def oracle_run(params, tensors, x_in, apply=offn.plain_ffn, autocast=False):
+        xr = x_in.clone().requires_grad_(True)
+        out = xr
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            for _ in range(4):
+                out = apply(out, params)
+        grads = torch.autograd.grad(_stack_objective(out.float()), [xr] + tensors)
+        return dict(zip(["out", "dx"] + names, [out.detach().float().cpu()] + [g.float().cpu() for g in grads]))
+
+    truth = oracle_run(p, [leaves[n] for n in names], x)
+    xd = x.to(DEV).requires_grad_(True)
+    out = xd
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=bf16):
+        for _ in range(4):
+            out = ffn(out)
+    params = dict(ffn.named_parameters())
+    grads = torch.autograd.grad(_stack_objective(out.float()), [xd] + [params[n] for n in names])
+    got = dict(zip(["out", "dx"] + names, [out.detach().float()] + list(grads)))
+    if not bf16:
+        for name in got:
+            assert_close(got[name], truth[name], dtype, name)
+        return
+    # bf16: four layers of rounding compound (without the residual nothing damps them), so the yard-stick is what stock-op
+    # bf16 runs of the same stack do: the oracle's plain composition and its memory-lean autograd.Function, under autocast
+    p_gpu, gpu_leaves = _oracle_with_named_leaves(ffn, device=DEV)
+    stock = [oracle_run(p_gpu, [gpu_leaves[n] for n in names], x.to(DEV), apply, autocast=True)
+             for apply in (offn.plain_ffn, offn.lean_ffn)]
+    assert_within_bf16_noise(got, truth, stock, "LeanFFN applied four times under bf16 autocast", depth=4)
+
+
+@pytest.mark.parametrize("layout,lowrank_dim,adapter_dim", [(None, 0, 0), ("pixelfly(16)", 4, 2), ("pixelfly(64)", 8, 0)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_two_layers_share_their_matrices(layout, lowrank_dim, adapter_dim, dtype):
+    """the reference builds its layers over shared GeneralizedMatrix objects (config.py:184-208: get_weight_matrix is cached
+    per key and matrix index): two LeanFFN layers with LayerNorms, biases and adapters of their own apply the same main
+    weights and low-rank factors.  The shared tensors' gradients are the sums over both layers; checked on the kernels
+    against the oracle with shared leaves."""
+    torch.manual_seed(7)
+    dim, inter = 128, 256
+    first = lt.GeneralizedMatrix(dim, 2 * inter, layout, lowrank_dim)
+    second = lt.GeneralizedMatrix(inter, dim, layout, lowrank_dim)
+    layers = [lt.LeanFFN(dim, inter, gated=True, layer_norm_eps=1e-5,
+                         i2h_proj=lt.GeneralizedLinear(first, adapter_dim), h2o_proj=lt.GeneralizedLinear(second, adapter_dim))
+              for _ in range(2)]
+    assert layers[0].i2h_proj.matrix is layers[1].i2h_proj.matrix and layers[0].h2o_proj.weight is layers[1].h2o_proj.weight
+    with torch.no_grad():
+        for i, ffn in enumerate(layers):
+            ffn.pre_layer_norm.weight.uniform_(0.5, 1.5)
+            ffn.pre_layer_norm.bias.normal_(std=0.2)
+            ffn.i2h_proj.bias.normal_(std=0.1)
+            for proj in (ffn.i2h_proj, ffn.h2o_proj):
+                if proj.adapter_second is not None:
+                    proj.adapter_second.normal_(std=0.1)
+    stack = nn.Sequential(*layers).to(DEV).to(dtype)
+    assert stack[0].i2h_proj.matrix.weight is stack[1].i2h_proj.matrix.weight  # still shared after the move and the cast
+    p0, leaves0 = _oracle_with_named_leaves(stack[0])
+    shared = {n: t for n, t in leaves0.items() if ".matrix." in n}
+    p1, leaves1 = _oracle_with_named_leaves(stack[1], shared)
+    x, dy = torch.randn(300, dim), torch.randn(300, dim)
+    xr = x.clone().requires_grad_(True)
+    y_ref = offn.plain_ffn(offn.plain_ffn(xr, p0), p1)
+    ref_leaves = {f"0.{n}": t for n, t in leaves0.items()}
+    ref_leaves.update({f"1.{n}": t for n, t in leaves1.items()})
+    named = dict(stack.named_parameters(remove_duplicate=False))
+    names = [n for n in named if not (n.startswith("1.") and ".matrix." in n)]  # each shared tensor once
+    ref = torch.autograd.grad(y_ref, [xr] + [ref_leaves[n] for n in names], dy)
+    xd = x.to(DEV).requires_grad_(True)
+    y = stack(xd)
+    got = torch.autograd.grad(y, [xd] + [named[n] for n in names], dy.to(DEV))
+    assert_close(y, y_ref.detach(), dtype, "y")
+    assert_close(got[0], ref[0], dtype, "dx")
+    for name, a, b in zip(names, got[1:], ref[1:]):
+        assert_close(a, b, dtype, name)
 
 
 @pytest.mark.parametrize("act", ["gelu_fused", "gelu", "relu", "silu"])

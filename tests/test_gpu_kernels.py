@@ -340,3 +340,48 @@ def test_empty_batch():
     assert layer(torch.empty(0, 32, device=DEV)).shape == (0, 64)
     ffn = lt.LeanFFN(32, 64).to(DEV)
     assert ffn(torch.empty(2, 0, 32, device=DEV)).shape == (2, 0, 32)
+
+
+def test_out_group_promise_is_checked_on_the_device_and_a_false_one_stays_inside_the_weight():
+    """lt_linear.out_group is a caller's promise about the index tables.  lt_linear_check_out_group tests it on the device;
+    a value that does not divide the number of output blocks is refused; and a false promise that passes that test makes the
+    forward kernel compute with the wrong blocks but never read outside the weight (NaNs sit right behind it here: the
+    results stay finite)."""
+    from lean_transformer_amd.blocksparse.linear import linear_desc
+    torch.manual_seed(3)
+    m = lt.GeneralizedMatrix(1024, 4096, "pixelfly(block_size=64, stretch=True)", 0).to(DEV).to(torch.bfloat16)
+    run = 4096 // 1024
+    fwd, bwd = m.forward_indices, m.backward_indices
+    lib = nat.lib()
+    flag = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    stream = nat.current_stream(flag.device)
+
+    def checked(group):
+        desc = linear_desc(m.weight.detach(), None, None, None, fwd, bwd)
+        desc.out_group = group
+        status = lib.lt_linear_check_out_group(desc, nat.ptr(flag), stream)
+        return status, (int(flag.item()) if status == 0 else None)
+
+    assert linear_desc(m.weight.detach(), None, None, None, fwd, bwd).out_group == run
+    assert checked(run) == (0, 1) and checked(2) == (0, 1) and checked(1) == (0, 1) and checked(0) == (0, 1)
+    assert checked(8) == (0, 0) and checked(16) == (0, 0)  # longer runs than the layout has
+    assert checked(3)[0] != 0 and "out_group" in lib.lt_last_error().decode()  # 64 output blocks are not a multiple of 3
+    # a false promise on the forward kernel (a square layout has no runs; runs of 4 are claimed): in bounds, finite, wrong
+    sq = lt.GeneralizedMatrix(2048, 2048, "pixelfly(block_size=64)", 0).to(DEV).to(torch.bfloat16)
+    assert linear_desc(sq.weight.detach(), None, None, None, sq.forward_indices, sq.backward_indices).out_group == 1
+    x = torch.randn(512, 2048, device=DEV).to(torch.bfloat16)
+    weight = torch.full((sq.weight.numel() + 65536,), float("nan"), dtype=torch.bfloat16, device=DEV)  # NaNs behind the weight
+    weight[:sq.weight.numel()] = sq.weight.detach().flatten()
+    w3 = weight[:sq.weight.numel()].view_as(sq.weight)
+    outs = []
+    for group in (1, 4):
+        desc = linear_desc(w3, None, None, None, sq.forward_indices, sq.backward_indices)
+        desc.out_group = group
+        y = torch.empty(512, 2048, dtype=torch.bfloat16, device=DEV)
+        nat.check(lib.lt_linear_forward(desc, 512, nat.dtype_code(torch.bfloat16), nat.ptr(x), nat.ptr(y), None, stream),
+                  "lt_linear_forward")
+        assert torch.isfinite(y.float()).all()
+        outs.append(y)
+    ref = obs.blocksparse_matmul(x.float().cpu(), sq.weight.detach().float().cpu(), sq.forward_indices.cpu().numpy())
+    assert_close(outs[0], ref, torch.bfloat16, "y without the promise")
+    assert not torch.equal(outs[0], outs[1])

@@ -90,3 +90,48 @@ def test_static_scratch_entry_allocates_nothing_and_refuses_what_does_not_fit():
                                nat.ptr(dx), None, None, nat.current_stream(dx.device)), "static without parameter gradients")
     torch.cuda.synchronize()
     assert torch.isfinite(dx).all()
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+from lean_transformer_amd import _native as nat
+dev = torch.device("cuda:0")
+tokens, hidden = 64, 256
+x = torch.randn(tokens, hidden, device=dev); dy = torch.randn(tokens, hidden, device=dev)
+w = torch.ones(hidden, device=dev); dx = torch.empty_like(x); dw = torch.empty(hidden, device=dev); db = torch.empty(hidden, device=dev)
+stats = torch.stack([x.mean(-1), torch.rsqrt(x.var(-1, unbiased=False) + 1e-5)], 1).contiguous()
+lib = nat.lib()
+def call(stream):
+    return lib.lt_layernorm_backward_static(tokens, hidden, 0, nat.ptr(x), nat.ptr(stats), nat.ptr(w), 0, nat.ptr(dy), 0, None,
+                                            nat.ptr(dx), nat.ptr(dw), nat.ptr(db), stream)
+side = torch.cuda.Stream()
+side.wait_stream(torch.cuda.current_stream())
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph, stream=side):
+    status = call(side.cuda_stream)          # first call on this device, on a capturing stream: refused, capture intact
+    dx.zero_()                               # (something for the graph to hold)
+assert status == 2 and b"outside stream capture" in lib.lt_last_error(), (status, lib.lt_last_error())
+graph.replay(); torch.cuda.synchronize()
+assert call(torch.cuda.current_stream().cuda_stream) == 0   # the warm-up call outside capture
+torch.cuda.synchronize()
+ref_dw = dw.clone()
+graph2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph2, stream=side):
+    assert call(side.cuda_stream) == 0       # now capturable
+dw.zero_(); graph2.replay(); torch.cuda.synchronize()
+assert torch.equal(dw, ref_dw)
+print("ok")
+"""
+
+
+def test_first_call_under_stream_capture_is_refused_and_later_calls_capture():
+    """the buffer's address is looked up on the first call on a device, which is not a stream operation: on a capturing stream
+    that first call is refused (and the capture survives); after one warm-up call the entry point captures and replays.
+    Needs a process in which the library has not been called yet: a child process."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", _FIRST_CALL_UNDER_CAPTURE, root], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "ok" in out.stdout, out.stdout + out.stderr
