@@ -23,6 +23,8 @@ def main():
     ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4"], help="bf16 benchmark configuration of bench.py")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--build", action="store_true", help="compile the instrumented library (hipcc, no GPU needed) and exit")
+    ap.add_argument("--distribution", action="store_true", help="dense configurations: also print how tile durations and "
+                    "end times spread over the tiles of each launch and over the eight XCDs (100 MHz real-time stamps)")
     args = ap.parse_args()
     root = os.path.dirname(os.path.abspath(__file__))
     sys.path.insert(0, root)
@@ -85,6 +87,20 @@ def main():
               f"{(loop.mean() - first16) / (ksteps - 16):6.1f})  epilogue {epilogue.mean():6.0f} (max {epilogue.max():6d})  "
               f"clock {clock:.3f} GHz")
     print(f"all six launches: matrix-core-ideal ticks / measured ticks = {total_ideal / total_ticks:.3f}")
+    if args.distribution:
+        import numpy as np
+        print("tile durations by the real-time counter (us); tile i of the launch order runs on XCD i % 8")
+        for (label, _), d in zip(launches, data):
+            idx = np.nonzero(d[:, 0])[0]
+            d = d[idx]
+            t0 = d[:, 4].min()
+            start, end = (d[:, 4] - t0) / 100.0, (d[:, 5] - t0) / 100.0
+            dur = end - start
+            last = idx >= len(idx) - min(256, len(idx))
+            per_xcd = " ".join(f"{dur[(idx & 7) == xcd].mean():6.1f}" for xcd in range(8))
+            print(f"{label:28s} duration min {dur.min():6.1f} p50 {np.median(dur):6.1f} p90 {np.percentile(dur, 90):6.1f} max {dur.max():6.1f}"
+                  f"  mean per XCD {per_xcd}  end of the last {int(last.sum())} tiles: min {end[last].min():6.1f} p50 "
+                  f"{np.median(end[last]):6.1f} max {end[last].max():6.1f}")
 
 
 def sparse_walks(torch, ffn, x, dy, params, cfg, dev):
