@@ -99,6 +99,15 @@ extern "C" int lt_linear_check_out_group(const lt_linear* lin, int32_t* flag, vo
   return LT_OK;
 }
 
+// Walk order of a block-sparse index list of `length` entries on the side with `many` blocks, seen from the side with `few`:
+// a stretched butterfly repeats every block of the square pattern many / few times in a row, so the lists are made of runs of
+// that many consecutive blocks (SparseWalk::walk_run; 0 when the shape suggests none).  Only an order: any layout computes right.
+int walk_run_for(int many, int few, int length) {
+  if (few <= 0 || many <= few || many % few != 0) return 0;
+  const int g = many / few;
+  return (g > 1 && length % g == 0) ? g : 0;
+}
+
 GemmOperand operand(const void* p, int64_t ld, bool kmajor) {
   GemmOperand o;
   o.ptr = p; o.ld = ld; o.kmajor = kmajor ? 1 : 0;
@@ -155,6 +164,7 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
   p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
   p.sp.backward_indices = lin.backward_indices; p.sp.act = x; p.sp.ld_act = in; p.sp.weight = lin.weight;
   p.sp.out_group = lin.out_group;
+  p.sp.walk_run = walk_run_for(lin.in_features / lin.block, lin.out_features / lin.block, lin.blocks_per_out);
   bool two_passes = gated && !(dtype == LT_BF16 && lt_sparse_mfma_supported(p, kind));
   if (gated && !two_passes) {
     // Gate and linear output blocks have index lists of their own; the bf16 walk for 64 x 64 blocks pairs them inside one
@@ -238,6 +248,7 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.mode = SPARSE_DX; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
       p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.weight = lin.weight;
+      p.sp.walk_run = walk_run_for(lin.out_features / lin.block, lin.in_features / lin.block, lin.blocks_per_in);
       if (kind_dx == EPI_ACT_BWD && act_colsum && (*act_colsum_rows = lt_gemm_colsum_rows(p, dtype, io_dtype)) > 0)
         p.epi.colsum = act_colsum;
       LT_TRY(lt_launch_gemm_sparse(p, kind_dx, dtype, io_dtype, stream));

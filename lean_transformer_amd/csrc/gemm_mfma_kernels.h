@@ -183,6 +183,12 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
       dw_ob[j] = sp.backward_indices[(int64_t)dw_ib * sp.blocks_per_in + min(dw_a0 + j, sp.blocks_per_in - 1)];
   }
 
+  // position in the group's index list taken at step t of the walk (see SparseWalk::walk_run)
+  auto walk_entry = [&](int t) {
+    if (sp.walk_run <= 1) return t;
+    const int runs = sp_steps / sp.walk_run;
+    return (t % runs) * sp.walk_run + t / runs;
+  };
   // global -> registers for k-step kt (ph: 0 = the tile's own block column, 1 = the matching linear block column)
   auto load_tiles = [&](int kt, int ph = 0) {
     const int seg = kt >= kt_seg0;
@@ -194,16 +200,17 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
     int64_t b_row0 = n0 + (PH == 2 ? ph * p.N : 0);  // first B row (k-major) / column (mn-major) of this tile
     if constexpr (SP == SPARSE_FWD) {
       if (!seg) {  // A: column block ib of X; B: weight block f, a [64 rows][64 k] matrix of its own
-        const int f = sp.forward_indices[(int64_t)(tn + (PH == 2 ? ph * tiles_n : 0)) * sp.blocks_per_out + kt];
+        const int f = sp.forward_indices[(int64_t)(tn + (PH == 2 ? ph * tiles_n : 0)) * sp.blocks_per_out + walk_entry(kt)];
         A = reinterpret_cast<const bf16*>(sp.act); lda = sp.ld_act; k0 = (int64_t)(f / sp.blocks_per_in) * 64;
         B = reinterpret_cast<const bf16*>(sp.weight) + (int64_t)f * 4096; ldb = 64; b_row0 = 0;
         K = k0 + 64;
       }
     } else if constexpr (SP == SPARSE_DX) {
       if (!seg) {  // A: column block ob of dY; B: weight block (ib, a) read as [64 k = output row][64 n = input column]
-        const int64_t ob = sp.backward_indices[(int64_t)tn * sp.blocks_per_in + kt];
+        const int a = walk_entry(kt);
+        const int64_t ob = sp.backward_indices[(int64_t)tn * sp.blocks_per_in + a];
         A = reinterpret_cast<const bf16*>(sp.act); lda = sp.ld_act; k0 = ob * 64;
-        B = reinterpret_cast<const bf16*>(sp.weight) + ((int64_t)tn * sp.blocks_per_in + kt) * 4096 - k0 * 64; ldb = 64;
+        B = reinterpret_cast<const bf16*>(sp.weight) + ((int64_t)tn * sp.blocks_per_in + a) * 4096 - k0 * 64; ldb = 64;
         b_row0 = 0;
         K = k0 + 64;
       }

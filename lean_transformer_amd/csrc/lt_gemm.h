@@ -67,6 +67,13 @@ struct SparseWalk {
   // With runs of 4 or more the weight gradient is computed on 256 x 256 tiles (4 output blocks x 4 input blocks of the
   // shared list), which read every dY column block once per 4 input blocks instead of once per input block.
   int out_group;
+  // FWD / DX walks (matrix-core kernel): order in which a group's index list is walked.  0 / 1: as listed.  g > 1 (must divide
+  // the list's length n): entry (t % (n / g)) * g + t / (n / g) at step t, i.e. the first members of the list's runs of g,
+  // then the second members, ...  In a stretched butterfly a list is made of runs of g consecutive blocks and the groups that
+  // share an activation block hold it at neighbouring positions of neighbouring runs: taken run-member by run-member they
+  // read it within a step or two of each other instead of g steps apart, while it is still in the XCD's L2.  Any g that
+  // divides n gives the same sums in another order; a g that fits no structure only costs what it would have gained.
+  int walk_run;
 };
 
 struct GemmProblem {
