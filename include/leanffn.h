@@ -84,7 +84,12 @@ typedef struct lt_linear {
                              kernels; 0 or 1 when not known, which is always safe.  Must divide the number of output blocks.
                              A false promise computes with the wrong weight blocks (it cannot make a kernel read outside
                              the weight); lt_linear_check_out_group tests it on the device. */
-  int32_t reserved;       /* 0 */
+  int32_t in_group;       /* sparse: every aligned run of this many consecutive input blocks has the same list of output
+                             blocks (backward_indices of input block ib0 + i = those of ib0).  PixelFly with stretch=True on
+                             a wide matrix: in_blocks / out_blocks.  A promise like out_group: it only selects a faster
+                             weight-gradient kernel, 0 or 1 is always safe, it must divide the number of input blocks, a false
+                             one puts wrong values into the weight gradient (never an access outside it), and
+                             lt_linear_check_in_group tests it on the device. */
 } lt_linear;
 
 /* Where lt_linear_backward / lt_ffn_backward write parameter gradients; a NULL member skips that gradient.
@@ -165,6 +170,8 @@ int lt_linear_backward(const lt_linear* lin, int64_t tokens, int32_t dtype, cons
  * like everything else: the caller reads the flag when it chooses (once per index table is enough).  No counterpart in the
  * reference, whose matmul takes no such hint. */
 int lt_linear_check_out_group(const lt_linear* lin, int32_t* flag, void* stream);
+/* The same for lin->in_group against lin->backward_indices.  No counterpart in the reference either. */
+int lt_linear_check_in_group(const lt_linear* lin, int32_t* flag, void* stream);
 
 /* ---- block-sparse matmul alone (weight in the native [in_features, A, block] format) ----------------------------------- */
 int lt_blocksparse_forward(const lt_linear* lin, int64_t tokens, int32_t dtype, const void* x, void* y, void* stream);

@@ -20,7 +20,7 @@ _DTYPES = {torch.float32: LT_F32, torch.bfloat16: LT_BF16}
 EXPORTED_SYMBOLS = (
     "lt_version", "lt_last_error",
     "lt_ffn_forward_workspace_bytes", "lt_ffn_backward_workspace_bytes", "lt_ffn_forward", "lt_ffn_backward",
-    "lt_linear_backward_workspace_bytes", "lt_linear_forward", "lt_linear_backward", "lt_linear_check_out_group",
+    "lt_linear_backward_workspace_bytes", "lt_linear_forward", "lt_linear_backward", "lt_linear_check_out_group", "lt_linear_check_in_group",
     "lt_blocksparse_forward", "lt_blocksparse_backward",
     "lt_layernorm_forward", "lt_layernorm_backward_workspace_bytes", "lt_layernorm_backward",
     "lt_layernorm_backward_static_scratch_bytes", "lt_layernorm_backward_static",
@@ -34,7 +34,7 @@ class LtLinear(ctypes.Structure):
         ("weight", c_void_p), ("bias", c_void_p), ("lowrank_first", c_void_p), ("lowrank_second", c_void_p),
         ("forward_indices", c_void_p), ("backward_indices", c_void_p),
         ("in_features", c_int32), ("out_features", c_int32), ("lowrank", c_int32), ("block", c_int32),
-        ("blocks_per_out", c_int32), ("blocks_per_in", c_int32), ("out_group", c_int32), ("reserved", c_int32),
+        ("blocks_per_out", c_int32), ("blocks_per_in", c_int32), ("out_group", c_int32), ("in_group", c_int32),
     ]
 
 
@@ -84,6 +84,7 @@ def _declare(lib):
     lib.lt_linear_backward_workspace_bytes.argtypes = [POINTER(LtLinear), c_int64, c_int32]
     lib.lt_linear_forward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.lt_linear_check_out_group.argtypes = [POINTER(LtLinear), c_void_p, c_void_p]
+    lib.lt_linear_check_in_group.argtypes = [POINTER(LtLinear), c_void_p, c_void_p]
     lib.lt_linear_backward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                        POINTER(LtLinearGrads), c_void_p, c_size_t, c_void_p]
     lib.lt_blocksparse_forward.argtypes = [POINTER(LtLinear), c_int64, c_int32, c_void_p, c_void_p, c_void_p]

@@ -164,12 +164,29 @@ def shared_list_run(forward_indices: torch.Tensor, blocks_per_in: int) -> int:
     return run
 
 
+def shared_input_run(backward_indices: torch.Tensor) -> int:
+    """The same on the input side: the largest power of two g such that every aligned run of g consecutive input blocks has
+    the same list of output blocks (PixelFly with ``stretch=True`` on a matrix with more input than output blocks: ``in_blocks
+    / out_blocks``).  Remembered on the tensor like shared_list_run."""
+    cached = getattr(backward_indices, "_lt_shared_input_run", None)
+    if cached is not None and cached[0] == backward_indices._version:
+        return cached[1]
+    run, n_in = 1, backward_indices.shape[0]
+    while n_in % (2 * run) == 0:
+        grouped = backward_indices.reshape(n_in // (2 * run), 2 * run, -1)
+        if not bool((grouped == grouped[:, :1]).all()):
+            break
+        run *= 2
+    backward_indices._lt_shared_input_run = (backward_indices._version, run)
+    return run
+
+
 def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices, backward_indices,
-                index_owner: Optional[torch.Tensor] = None) -> "nat.LtLinear":
-    """ctypes descriptor of one projection; all tensors already in their final dtype and contiguous.  index_owner: the
-    caller's own forward_indices tensor (the module's buffer) when `forward_indices` may be a converted copy of it: the
-    shared-list run is remembered on that object, so that a copy made per call does not recompute it (and synchronise) per
-    call."""
+                index_owner: Optional[torch.Tensor] = None, backward_owner: Optional[torch.Tensor] = None) -> "nat.LtLinear":
+    """ctypes descriptor of one projection; all tensors already in their final dtype and contiguous.  index_owner /
+    backward_owner: the caller's own forward_indices / backward_indices tensors (the module's buffers) when the ones passed
+    may be converted copies of them: the shared-list runs are remembered on those objects, so that a copy made per call
+    does not recompute them (and synchronise) per call."""
     desc = nat.LtLinear()
     desc.weight = nat.ptr(weight)
     desc.bias = nat.ptr(bias_f32)
@@ -187,6 +204,8 @@ def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices
         desc.out_group = shared_list_run(owner, blocks_per_in)
         if desc.out_group > 1 and forward_indices.shape[0] % desc.out_group:
             desc.out_group = 1  # (cannot happen for a power of two that divides the block count; the C ABI refuses it)
+        if backward_indices is not None:
+            desc.in_group = shared_input_run(backward_indices if backward_owner is None else backward_owner)
     return desc
 
 
@@ -210,7 +229,7 @@ class _GeneralizedLinear(torch.autograd.Function):
         b32 = _as(bias, torch.float32)
         fwd = None if forward_indices is None else forward_indices.to(torch.int32).contiguous()
         bwd = None if backward_indices is None else backward_indices.to(torch.int64).contiguous()
-        desc = linear_desc(w, b32, l1, l2, fwd, bwd, forward_indices)
+        desc = linear_desc(w, b32, l1, l2, fwd, bwd, forward_indices, backward_indices)
         if x.shape[1] != desc.in_features:
             raise ValueError(f"input has {x.shape[1]} features, the weight takes {desc.in_features}")
         tokens = x.shape[0]
@@ -235,7 +254,7 @@ class _GeneralizedLinear(torch.autograd.Function):
         l1, l2 = _as(lowrank_first, dtype), _as(lowrank_second, dtype)
         fwd = None if forward_indices is None else forward_indices.to(torch.int32).contiguous()
         bwd = None if backward_indices is None else backward_indices.to(torch.int64).contiguous()
-        desc = linear_desc(w, None, l1, l2, fwd, bwd, forward_indices)
+        desc = linear_desc(w, None, l1, l2, fwd, bwd, forward_indices, backward_indices)
         tokens = x.shape[0]
         grads = nat.LtLinearGrads()
         dx = torch.empty_like(x) if need[0] else None

@@ -66,6 +66,8 @@ int check_linear(const lt_linear& lin, const char* name, int tables = NEED_FWD_T
                LT_ERR_BAD_ARG, "%s: unbalanced layout (K=%d, A=%d)", name, lin.blocks_per_out, lin.blocks_per_in);
     LT_REQUIRE(lin.out_group >= 0 && (lin.out_group <= 1 || (lin.out_features / lin.block) % lin.out_group == 0), LT_ERR_BAD_ARG,
                "%s: out_group=%d does not divide the %d output blocks", name, lin.out_group, lin.out_features / lin.block);
+    LT_REQUIRE(lin.in_group >= 0 && (lin.in_group <= 1 || (lin.in_features / lin.block) % lin.in_group == 0), LT_ERR_BAD_ARG,
+               "%s: in_group=%d does not divide the %d input blocks", name, lin.in_group, lin.in_features / lin.block);
   }
   return LT_OK;
 }
@@ -81,6 +83,14 @@ __global__ void check_out_group_kernel(const int32_t* __restrict__ forward_indic
   const int mine = forward_indices[i], first = forward_indices[ob0 * per_out + e];
   if (mine / per_in != first / per_in || mine != first + (ob - ob0)) flag[0] = 0;
 }
+// the same for lt_linear::in_group: input block ib's list of output blocks against that of the first block of its run
+__global__ void check_in_group_kernel(const int64_t* __restrict__ backward_indices, int in_blocks, int per_in, int group,
+                                      int32_t* flag) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= in_blocks * per_in) return;
+  const int ib = i / per_in, e = i % per_in, ib0 = ib - ib % group;
+  if (backward_indices[i] != backward_indices[ib0 * per_in + e]) flag[0] = 0;
+}
 __global__ void set_flag_kernel(int32_t* flag, int32_t value) { flag[0] = value; }
 }  // namespace
 
@@ -94,6 +104,21 @@ extern "C" int lt_linear_check_out_group(const lt_linear* lin, int32_t* flag, vo
     const int out_blocks = lin->out_features / lin->block, entries = out_blocks * lin->blocks_per_out;
     hipLaunchKernelGGL(check_out_group_kernel, dim3((unsigned)((entries + 255) / 256)), dim3(256), 0, stream,
                        lin->forward_indices, out_blocks, lin->blocks_per_out, lin->blocks_per_in, lin->out_group, flag);
+    LT_LAUNCH_CHECK();
+  }
+  return LT_OK;
+}
+
+extern "C" int lt_linear_check_in_group(const lt_linear* lin, int32_t* flag, void* stream_) {
+  LT_REQUIRE(lin && flag, LT_ERR_BAD_ARG, "check in_group: null argument");
+  LT_TRY(check_linear(*lin, "check in_group", NEED_BWD_TABLE));
+  hipStream_t stream = (hipStream_t)stream_;
+  hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, stream, flag, 1);
+  LT_LAUNCH_CHECK();
+  if (lin->block > 0 && lin->in_group > 1) {
+    const int in_blocks = lin->in_features / lin->block, entries = in_blocks * lin->blocks_per_in;
+    hipLaunchKernelGGL(check_in_group_kernel, dim3((unsigned)((entries + 255) / 256)), dim3(256), 0, stream,
+                       lin->backward_indices, in_blocks, lin->blocks_per_in, lin->in_group, flag);
     LT_LAUNCH_CHECK();
   }
   return LT_OK;
@@ -203,6 +228,8 @@ void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, 
     if (lin.lowrank == 0)
       s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_generic_splitk_workspace(T, lin.in_features, lin.out_features));
   }
+  if (lin.block == 64 && dtype == LT_BF16)
+    s.skinny_bytes = std::max(s.skinny_bytes, lt_sparse_dw_split_workspace(lin.in_features, lin.blocks_per_in, lin.in_group, T));
   s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 
@@ -270,8 +297,23 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.act2 = x_act;
       p.sp.ld_act2 = in; p.sp.tokens = T;
       p.sp.out_group = lin.forward_indices ? lin.out_group : 0;  // the grouped kernel reads the list from the forward table
+      p.sp.in_group = lin.in_group;
       p.epi = epi_store_params(grads.weight, lin.block, dtype, nullptr);
-      LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));
+      const int slices = dtype == LT_BF16 ? lt_sparse_dw_in_grouped_slices(p) : 0;
+      const size_t elements = (size_t)(in / lin.block) * lin.blocks_per_in * lin.block * lin.block;
+      if (slices > 1 && s.skinny && s.skinny_bytes >= (size_t)slices * elements * sizeof(float)) {
+        // the reduction over the tokens split over workgroups: fp32 partial gradients, summed into the parameter's dtype
+        p.ksplit = slices;
+        p.split_stride = (int64_t)elements;
+        p.epi.out = s.skinny;
+        p.epi.out_dtype = LT_F32;
+        LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));
+        LT_TRY(lt_splitk_reduce((const float*)s.skinny, slices, (int64_t)elements, (int64_t)elements, lin.block, nullptr, dtype,
+                                grads.weight, stream));
+      } else {
+        if (slices > 1) p.sp.in_group = 0;  // no room for the partial sums: the walk
+        LT_TRY(lt_launch_gemm_sparse(p, EPI_STORE, dtype, io_dtype, stream));
+      }
     }
   }
   if (r > 0 && grads.lowrank_second) {  // dL2[out, r] = dy^T hid

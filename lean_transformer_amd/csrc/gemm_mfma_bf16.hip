@@ -306,6 +306,36 @@ bool lt_sparse_forward_grouped(const GemmProblem& p, int kind) {
   return true;
 }
 
+bool lt_sparse_dw_out_grouped(const GemmProblem& p) {
+  const SparseWalk& sp = p.sp;
+  const int64_t out_features = sp.ld_act;
+  return sp.mode == SPARSE_DW && sp.out_group >= 4 && sp.out_group % 4 == 0 && sp.forward_indices && out_features % 256 == 0 &&
+         sp.tokens % DK == 0 && sp.tokens > 0 && 32 * sp.ld_act * 2 + out_features * 2 < (int64_t)1 << 32 &&
+         32 * sp.ld_act2 * 2 + p.N * 2 < (int64_t)1 << 32;
+}
+
+int lt_sparse_dw_in_grouped_slices(const GemmProblem& p) {
+  const SparseWalk& sp = p.sp;
+  const int64_t out_features = sp.ld_act, in_features = p.N;
+  if (sp.mode != SPARSE_DW || !lt_sparse_mfma_supported(p, EPI_STORE) || lt_sparse_dw_out_grouped(p)) return 0;
+  if (sp.in_group < 4 || sp.in_group % 4 != 0 || !sp.backward_indices || in_features % 256 != 0) return 0;
+  if (sp.tokens <= 0 || sp.tokens % DK != 0) return 0;
+  if (32 * sp.ld_act * 2 + out_features * 2 >= (int64_t)1 << 32 || 32 * sp.ld_act2 * 2 + in_features * 2 >= (int64_t)1 << 32) return 0;
+  // enough workgroups for the 256 CUs, each slice at least 32 k-steps long
+  const int64_t tiles = (int64_t)((sp.blocks_per_in + 3) / 4) * (in_features / 256);
+  if (tiles >= 192) return 1;
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, sp.tokens / (32 * DK)), 8));
+}
+
+size_t lt_sparse_dw_split_workspace(int64_t in_features, int blocks_per_in, int in_group, int64_t tokens) {
+  if (in_group < 4 || in_features % 256 != 0) return 0;
+  // (an upper bound that needs no more than the layer's shape: 8 slices at most)
+  const int64_t tiles = (int64_t)((blocks_per_in + 3) / 4) * (in_features / 256);
+  if (tiles >= 192) return 0;
+  const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, tokens / (32 * DK)), 8));
+  return slices > 1 ? lt_align_up((size_t)slices * (size_t)(in_features / 64) * blocks_per_in * 4096 * sizeof(float), 256) : 0;
+}
+
 int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream) {
   if (dtype != LT_BF16 || !lt_sparse_mfma_supported(p, kind)) return lt_launch_gemm_generic(p, kind, dtype, io_dtype, stream);
   const SparseWalk& sp = p.sp;

@@ -99,11 +99,15 @@ template <int N, typename F> __device__ __forceinline__ void lt_static_for(F&& f
 // linear block tn + N / 64, which have index lists of their own.  It walks the two lists one after the other (two phases
 // over the same LDS stages) into two sets of accumulators and pairs them in the epilogue, so the gated activation needs no
 // pass of its own over the pre-activations.
-template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX, int SP = SPARSE_NONE, int PH = 1>
+// PF: how many k-steps ahead of the matrix instructions the operand tiles are requested (in registers; the LDS holds two
+// stages whatever PF is).  1 for the MFMA-bound uses; the rank-r products stream a large operand once against a small one and
+// are bound by how many bytes a CU has in flight, so they ask further ahead.
+template <int BM, int BN, int WM, int WN, bool A_KM, bool B_KM, int KIND, typename TX, int SP = SPARSE_NONE, int PH = 1, int PF = 1>
 __global__ __launch_bounds__(WM * WN * 64)
-__attribute__((amdgpu_waves_per_eu(SP != SPARSE_NONE ? 2 : 1)))  // the block-sparse walks: two workgroups per CU (their LDS allows it)
+__attribute__((amdgpu_waves_per_eu((SP != SPARSE_NONE || PF > 1) ? 2 : 1)))  // block-sparse walks, rank-r products: two workgroups per CU
 void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int NT = WM * WN * 64;
+  static_assert(PF == 1 || (SP == SPARSE_NONE && PH == 1), "deeper prefetch: dense single-phase only");
   static_assert(PH == 1 || (PH == 2 && SP == SPARSE_FWD && KIND == EPI_ACT_FWD && WN == 1), "two phases: gated block-sparse forward");
   static_assert(SP == SPARSE_NONE || (SP == SPARSE_FWD && A_KM && B_KM && BN == 64) ||
                     (SP == SPARSE_DX && A_KM && !B_KM && BN == 64) ||
@@ -160,7 +164,7 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  u32x4 ra[A_CHUNKS], rb[B_CHUNKS];
+  u32x4 ra_set[PF][A_CHUNKS], rb_set[PF][B_CHUNKS];
 
   // k-steps: dense: segment 0 then segment 1; sparse FWD / DX: the active blocks of this group, then the low-rank segment
   const SparseWalk& sp = p.sp;
@@ -190,7 +194,7 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
     return (t % runs) * sp.walk_run + t / runs;
   };
   // global -> registers for k-step kt (ph: 0 = the tile's own block column, 1 = the matching linear block column)
-  auto load_tiles = [&](int kt, int ph = 0) {
+  auto load_tiles = [&](int kt, int ph, u32x4 (&ra)[A_CHUNKS], u32x4 (&rb)[B_CHUNKS]) __attribute__((always_inline)) {
     const int seg = kt >= kt_seg0;
     int64_t k0 = (int64_t)(seg ? kt - kt_seg0 : kt) * BK;
     int64_t K = p.K[seg];
@@ -227,11 +231,13 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
         const int64_t gm = min(m0 + row, p.M - 1);  // rows past M are clamped (their results are never stored)
         ra[i] = *reinterpret_cast<const u32x4*>(A + gm * lda + k0 + c * 8);
       } else {
+        // rows past K: the last row again, zeroed on the way into LDS (store_tiles) -- a load under a branch would make
+        // every later wait on the memory counter a wait for all of them, and no load could stay in flight across a step
         const int kr = q / (BM / 8), c = q % (BM / 8);
-        const int64_t gk = k0 + kr;
+        const int64_t gk = min(k0 + kr, K - 1);
         int64_t col = m0 + c * 8;
         if constexpr (SP == SPARSE_DW) col = dw_ob[c >> 3] * 64 + (c & 7) * 8;
-        ra[i] = gk < K ? *reinterpret_cast<const u32x4*>(A + gk * lda + col) : u32x4{0u, 0u, 0u, 0u};
+        ra[i] = *reinterpret_cast<const u32x4*>(A + gk * lda + col);
       }
     }
 #pragma unroll
@@ -251,22 +257,30 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
         rb[i] = *reinterpret_cast<const u32x4*>(B + gn * ldb + bk0 + c * 8);
       } else {
         const int kr = q / (BN / 8), c = q % (BN / 8);
-        const int64_t gk = k0 + kr;
-        rb[i] = gk < K ? *reinterpret_cast<const u32x4*>(B + gk * ldb + b_row0 + c * 8) : u32x4{0u, 0u, 0u, 0u};
+        const int64_t gk = min(k0 + kr, K - 1);
+        rb[i] = *reinterpret_cast<const u32x4*>(B + gk * ldb + b_row0 + c * 8);
       }
     }
   };
+  // how many of the BK k-rows of step kt exist; mn-major operand tiles are zero-filled past them
+  auto k_rows = [&](int kt) -> int {
+    const int seg = kt >= kt_seg0;
+    if ((SP == SPARSE_FWD || SP == SPARSE_DX) && !seg) return BK;
+    const int64_t k0 = (int64_t)(seg ? kt - kt_seg0 : kt) * BK;
+    const int64_t K = SP == SPARSE_DW ? (int64_t)sp.tokens : p.K[seg];
+    return (int)min((int64_t)BK, K - k0);
+  };
   // registers -> LDS stage s
-  auto store_tiles = [&](int s) {
+  auto store_tiles = [&](int s, int rows, const u32x4 (&ra)[A_CHUNKS], const u32x4 (&rb)[B_CHUNKS]) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; i++) {
       const int q = tid + i * NT;
       if constexpr (A_KM) {
         const int row = q >> 3, c = q & 7;
-        *reinterpret_cast<u32x4*>(&lds_a[s][(row * 8 + (c ^ swz_km(row))) * 8]) = ra[i];
+        *reinterpret_cast<u32x4*>(&lds_a[s][(row * 8 + (c ^ swz_km(row))) * 8]) = (PF == 1 || rows > 0) ? ra[i] : u32x4{0u, 0u, 0u, 0u};
       } else {
         const int kr = q / (BM / 8), c = q % (BM / 8);
-        *reinterpret_cast<u32x4*>(&lds_a[s][kr * BM + ((c ^ swz_mn_cols<BM>(kr)) << 3)]) = ra[i];
+        *reinterpret_cast<u32x4*>(&lds_a[s][kr * BM + ((c ^ swz_mn_cols<BM>(kr)) << 3)]) = kr < rows ? ra[i] : u32x4{0u, 0u, 0u, 0u};
       }
     }
 #pragma unroll
@@ -274,10 +288,10 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
       const int q = tid + i * NT;
       if constexpr (B_KM) {
         const int row = q >> 3, c = q & 7;
-        *reinterpret_cast<u32x4*>(&lds_b[s][(row * 8 + (c ^ swz_km(row))) * 8]) = rb[i];
+        *reinterpret_cast<u32x4*>(&lds_b[s][(row * 8 + (c ^ swz_km(row))) * 8]) = (PF == 1 || rows > 0) ? rb[i] : u32x4{0u, 0u, 0u, 0u};
       } else {
         const int kr = q / (BN / 8), c = q % (BN / 8);
-        *reinterpret_cast<u32x4*>(&lds_b[s][kr * BN + ((c ^ swz_mn_cols<BN>(kr)) << 3)]) = rb[i];
+        *reinterpret_cast<u32x4*>(&lds_b[s][kr * BN + ((c ^ swz_mn_cols<BN>(kr)) << 3)]) = kr < rows ? rb[i] : u32x4{0u, 0u, 0u, 0u};
       }
     }
   };
@@ -340,22 +354,59 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
     }
   };
   LT_TILE_STAMP(1);
-  lt_static_for<PH>([&](auto PHASE) __attribute__((always_inline)) {
-    constexpr int ph = decltype(PHASE)::value;
-    if (kt_begin < kt_end) {
-      load_tiles(kt_begin, ph);
-      store_tiles(kt_begin & 1);
-    }
-    __syncthreads();
-    for (int kt = kt_begin; kt < kt_end; kt++) {
-      const int s = kt & 1;
-      const bool has_next = kt + 1 < kt_end;
-      if (has_next) load_tiles(kt + 1, ph);
-      multiply_stage(s, PHASE);
-      if (has_next) store_tiles(s ^ 1);
+  if constexpr (PF == 1) {
+    lt_static_for<PH>([&](auto PHASE) __attribute__((always_inline)) {
+      constexpr int ph = decltype(PHASE)::value;
+      if (kt_begin < kt_end) {
+        load_tiles(kt_begin, ph, ra_set[0], rb_set[0]);
+        store_tiles(kt_begin & 1, k_rows(kt_begin), ra_set[0], rb_set[0]);
+      }
       __syncthreads();
+      for (int kt = kt_begin; kt < kt_end; kt++) {
+        const int s = kt & 1;
+        const bool has_next = kt + 1 < kt_end;
+        if (has_next) load_tiles(kt + 1, ph, ra_set[0], rb_set[0]);
+        multiply_stage(s, PHASE);
+        if (has_next) store_tiles(s ^ 1, k_rows(kt + 1), ra_set[0], rb_set[0]);
+        __syncthreads();
+      }
+    });
+  } else {
+    // Register set d holds step i with i % PF == d from its request until it is written to LDS stage i & 1 at the end of
+    // step i - 1; the set is then free for step i + PF, requested at the start of step i.
+    // A k-major operand with a power-of-two row pitch: the 128 rows of a tile, and the same k-step of every tile row, sit
+    // on the same memory channels, so tile row tm starts its walk over the slice tm steps in and wraps around.
+    // Nothing in the loop is conditional (a load or an LDS write under a branch makes every later wait on the memory counter
+    // a wait for all loads): the walk is padded to a multiple of PF steps, requests past its end repeat the last tile and
+    // such a tile is written to LDS as zeros.
+    const int steps = kt_end - kt_begin;
+    if (steps > 0) {
+      const int padded = (steps + PF - 1) / PF * PF;
+      const int rot = (A_KM && steps > 1) ? tm % steps : 0;
+      auto kt_of = [&](int i) {
+        const int j = min(i, steps - 1) + rot;
+        return kt_begin + (j >= steps ? j - steps : j);
+      };
+      auto rows_of = [&](int i) { return i < steps ? k_rows(kt_of(i)) : 0; };
+      lt_static_for<PF>([&](auto D) __attribute__((always_inline)) {
+        constexpr int d = decltype(D)::value;
+        load_tiles(kt_of(d), 0, ra_set[d], rb_set[d]);
+      });
+      store_tiles(0, rows_of(0), ra_set[0], rb_set[0]);
+      __syncthreads();
+      for (int i0 = 0; i0 < padded; i0 += PF) {
+        lt_static_for<PF>([&](auto D) __attribute__((always_inline)) {
+          constexpr int d = decltype(D)::value;
+          const int i = i0 + d;
+          const int s = i & 1;
+          load_tiles(kt_of(i + PF), 0, ra_set[d], rb_set[d]);
+          multiply_stage(s, std::integral_constant<int, 0>{});
+          store_tiles(s ^ 1, rows_of(i + 1), ra_set[(d + 1) % PF], rb_set[(d + 1) % PF]);
+          __syncthreads();
+        });
+      }
     }
-  });
+  }
   LT_TILE_STAMP(2);
 
   // ---- epilogue.  The accumulators of a 32 x 32 block sit column-per-lane (register r = row 8 * (r / 4) + 4 * (lane / 32)
@@ -758,7 +809,9 @@ constexpr bool SPLIT_MN_B = true;
 // SCATTER (EPI_STORE only; the grouped block-sparse weight gradient): the tile is 4 output blocks (rows) x 4 entries of
 // their shared list of input blocks (columns); each 64 x 64 piece goes to its own block of the native [in, A, block] weight
 // gradient, at the flat position the forward table names.  List entries past the end (the last column tile) are not stored.
-template <int FM, int KIND, typename TX, int tile_rows, int tile_cols, bool SCATTER = false>
+// SCATTER == 2: the tile is 4 entries of a list of output blocks (rows) x the run of 4 input blocks that shares the list
+// (columns); piece (entry a, input block ib) is block ib * blocks_per_in + a.
+template <int FM, int KIND, typename TX, int tile_rows, int tile_cols, int SCATTER = 0>
 __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const GemmProblem& p, float* stage, const int64_t m0,
                                                   const int64_t n0, const int wm, const int wn, const bool gated) {
   constexpr int FN = 4, WTN = 128, WTM = FM * 32;
@@ -939,10 +992,19 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
     constexpr int i = decltype(I)::value;
     constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_IT = 64 / LANES_PER_ROW, NIT = 32 / ROWS_PER_IT;
     const int c = (lane % LANES_PER_ROW) * 8;
-    const int per_out = p.sp.blocks_per_out;
-    const int64_t ob = m0 / 64 + (wm * WTM + i * 32) / 64;
-    const int entry = (int)(n0 / 64) + wn * 2 + (c >> 6);  // position in the output block's list
-    const int64_t flat = p.sp.forward_indices[ob * per_out + min(entry, per_out - 1)];
+    int per_out, entry;  // length of the list, position in it
+    int64_t flat;
+    if constexpr (SCATTER == 1) {
+      per_out = p.sp.blocks_per_out;
+      const int64_t ob = m0 / 64 + (wm * WTM + i * 32) / 64;
+      entry = (int)(n0 / 64) + wn * 2 + (c >> 6);
+      flat = p.sp.forward_indices[ob * per_out + min(entry, per_out - 1)];
+    } else {
+      per_out = p.sp.blocks_per_in;
+      entry = (int)(m0 / 64) + (wm * WTM + i * 32) / 64;
+      const int64_t ib = n0 / 64 + wn * 2 + (c >> 6);
+      flat = ib * per_out + min(entry, per_out - 1);
+    }
     TO* dst = reinterpret_cast<TO*>(epi.out) + flat * 4096 + ((i & 1) * 32 + lane / LANES_PER_ROW) * 64 + (c & 63);
     stage_strip(I);
     float v[NIT][8];
@@ -953,7 +1015,7 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
     }
     __builtin_amdgcn_wave_barrier();
   };
-  if constexpr (SCATTER) {
+  if constexpr (SCATTER != 0) {
     static_assert(KIND == EPI_STORE, "scattered blocks: plain store");
     if (epi.out_dtype == LT_F32) for_each_strip([&](auto I) { scatter_strip(I, float{}); });
     else for_each_strip([&](auto I) { scatter_strip(I, bf16{}); });
@@ -1014,6 +1076,10 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
 // GATHER == 1 (both operands mn-major, plain store): the weight gradient.  A = dY [tokens, out], a tile row = a run of 4
 //   output blocks; B = X [tokens, in], a tile column = 4 entries of the run's list, gathered as four 64-wide column blocks;
 //   the result is scattered to the weight gradient's blocks (SCATTER above).
+// GATHER == 3 (both operands mn-major, plain store): the weight gradient of a layout whose runs are on the input side (every
+//   aligned run of 4 consecutive input blocks has the same list of output blocks).  A = dY, a tile row = 4 entries of the
+//   run's list, gathered as four 64-wide column blocks; B = X, a tile column = the run of 4 input blocks; the 64 x 64 piece
+//   (entry a, input block ib) is weight-gradient block ib * blocks_per_in + a.
 // GATHER == 2 (both operands k-major): the forward product.  A tile column = a run of 4 output blocks; k-block e of the first
 //   k-segment is entry e of the run's list: A = column block ib_e of X, B = the four weight blocks (ib_e, a_e .. a_e + 3),
 //   which are adjacent in the native [in, A, block] layout (the run's blocks are consecutive among the active output blocks of
@@ -1033,7 +1099,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
   typedef const __attribute__((address_space(4))) GemmProblem* KernargProblem;
   KernargProblem pk = (KernargProblem)__builtin_amdgcn_kernarg_segment_ptr();
 #define p (*pk)
-  static_assert(GATHER != 1 || (!A_KM && !B_KM && KIND == EPI_STORE && !K_TAIL), "gathered columns: weight-gradient layout");
+  static_assert((GATHER != 1 && GATHER != 3) || (!A_KM && !B_KM && KIND == EPI_STORE && !K_TAIL), "gathered columns: weight-gradient layout");
   static_assert(GATHER != 2 || (A_KM && B_KM && !K_TAIL), "gathered k-blocks: forward layout");
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128, FM = 4, FN = 4;
   constexpr int HALF = 4;  // copy instructions per wavefront for a mn-major k-step or half a k-major block
@@ -1167,6 +1233,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
     if (GATHER == 2 && seg == 0) {
       const GemmOperand x = {p.sp.act, p.sp.ld_act, 1};
       ca.setup(x, 0, m0, p.M, 0, wave, lane);  // unit u = column block u of X
+    } else if constexpr (GATHER == 3) {
+      // the output blocks of list entries tm * 4 .. tm * 4 + 3 of input block tn * 4 (past the end: the last entry again)
+      int blocks[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int entry = min(tm * 4 + j, p.sp.blocks_per_in - 1);
+        blocks[j] = (int)p.sp.backward_indices[(int64_t)tn * 4 * p.sp.blocks_per_in + entry];
+      }
+      const GemmOperand a = {p.A[0].ptr, p.A[0].ld, p.A[0].kmajor};
+      ca.setup_gather(a, blocks, wave, lane);
     } else {
       const GemmOperand a = {p.A[seg].ptr, p.A[seg].ld, p.A[seg].kmajor};
       ca.setup(a, seg, m0, p.M, 0, wave, lane);
@@ -1462,7 +1538,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
                             : wave == 1 ? (A_KM ? a_d1 + KM_ELEMS / 2 : a_s3)
                             : wave == 2 ? (B_KM ? b_d1 : b_s2)
                                         : (B_KM ? b_d1 + KM_ELEMS / 2 : b_s3);
-    dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER == 1>(acc, *(const GemmProblem*)pk, reinterpret_cast<float*>(stage_buf), epi_m0,
+    dma_tile_epilogue<FM, KIND, TX, BM, BN, GATHER == 1 ? 1 : GATHER == 3 ? 2 : 0>(acc, *(const GemmProblem*)pk, reinterpret_cast<float*>(stage_buf), epi_m0,
                                                           epi_n0, wm, wn, gated);
     LT_TILE_STAMP(3);
     LT_TILE_STAMP_REALTIME(5);
@@ -1596,8 +1672,7 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
   } else {
     if constexpr (KIND == EPI_STORE) {
       const int64_t out_features = sp.ld_act;
-      if (sp.out_group >= 4 && sp.out_group % 4 == 0 && sp.forward_indices && out_features % 256 == 0 && sp.tokens % DK == 0 &&
-          sp.tokens > 0 && 32 * sp.ld_act * 2 + out_features * 2 < (int64_t)1 << 32 && 32 * sp.ld_act2 * 2 + p.N * 2 < (int64_t)1 << 32) {
+      if (lt_sparse_dw_out_grouped(p)) {
         // grouped: a dense both-operands-mn-major product dY^T X per run of 4 output blocks, over their shared list
         GemmProblem q = p;
         q.M = out_features;
@@ -1609,6 +1684,22 @@ template <int KIND> int launch_sparse(const GemmProblem& problem, int io_dtype, 
         q.ksplit = 0; q.krot = 0;
         hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, 1>), dim3(dma_grid(q, tiles_m * tiles_n)),
                            block, 0, stream, q, tiles_m, tiles_n);
+        LT_LAUNCH_CHECK();
+        return LT_OK;
+      }
+      if (lt_sparse_dw_in_grouped_slices(p) > 0) {
+        // grouped on the input side: dY^T X per run of 4 input blocks, over their shared list of output blocks.  The
+        // reduction is split only when the caller asked (p.ksplit slices, epi.out pointing at fp32 partial sums)
+        const int slices = p.ksplit > 1 ? p.ksplit : 1;
+        GemmProblem q = p;
+        const int tiles_m = (sp.blocks_per_in + 3) / 4, tiles_n = (int)(p.N / 256);
+        q.M = (int64_t)tiles_m * 256;
+        q.nseg = 1; q.K[0] = sp.tokens; q.K[1] = 0;
+        q.A[0].ptr = sp.act; q.A[0].ld = sp.ld_act; q.A[0].kmajor = 0;
+        q.B[0].ptr = sp.act2; q.B[0].ld = sp.ld_act2; q.B[0].kmajor = 0;
+        q.ksplit = slices > 1 ? slices : 0; q.krot = 0;
+        hipLaunchKernelGGL((gemm_bf16_dma_kernel<false, false, EPI_STORE, float, false, 3>),
+                           dim3(dma_grid(q, tiles_m * tiles_n), (unsigned)slices), block, 0, stream, q, tiles_m, tiles_n);
         LT_LAUNCH_CHECK();
         return LT_OK;
       }

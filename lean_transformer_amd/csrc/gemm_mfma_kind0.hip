@@ -13,7 +13,8 @@ namespace {
 template <bool A_KM, bool B_KM> int launch_skinny(const GemmProblem& p, int slices, hipStream_t stream) {
   const int tiles_m = (int)((p.M + 127) / 128), tiles_n = (int)(p.N / 128);
   dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)slices), block(256);
-  hipLaunchKernelGGL((gemm_bf16_kernel<128, 128, 2, 2, A_KM, B_KM, EPI_STORE, float>), grid, block, 0, stream, p, tiles_m, tiles_n);
+  // these products stream one large operand once against a small one: operand tiles are requested two k-steps ahead
+  hipLaunchKernelGGL((gemm_bf16_kernel<128, 128, 2, 2, A_KM, B_KM, EPI_STORE, float, SPARSE_NONE, 1, 2>), grid, block, 0, stream, p, tiles_m, tiles_n);
   LT_LAUNCH_CHECK();
   return LT_OK;
 }

@@ -67,6 +67,10 @@ struct SparseWalk {
   // With runs of 4 or more the weight gradient is computed on 256 x 256 tiles (4 output blocks x 4 input blocks of the
   // shared list), which read every dY column block once per 4 input blocks instead of once per input block.
   int out_group;
+  // DW: every aligned run of this many consecutive input blocks shares one list of output blocks (0 / 1: not known to).  With
+  // runs of 4 or more, and none on the output side, the weight gradient runs on 256 x 256 tiles of 4 list entries x 4 input
+  // blocks.
+  int in_group;
   // FWD / DX walks (matrix-core kernel): order in which a group's index list is walked.  0 / 1: as listed.  g > 1 (must divide
   // the list's length n): entry (t % (n / g)) * g + t / (n / g) at step t, i.e. the first members of the list's runs of g,
   // then the second members, ...  In a stretched butterfly a list is made of runs of g consecutive blocks and the groups that
@@ -473,6 +477,13 @@ double lt_gemm_flops(const GemmProblem& p, int kind);
 // whether a block-sparse forward problem (plain store or non-gated activation epilogue) runs as a dense product over
 // gathered k-blocks: its output blocks come in aligned runs of 4 or more that share one list of input blocks (sp.out_group)
 bool lt_sparse_forward_grouped(const GemmProblem& p, int kind);
+// whether a block-sparse weight-gradient problem (SPARSE_DW) runs as dense products per run of 4 output blocks (sp.out_group)
+bool lt_sparse_dw_out_grouped(const GemmProblem& p);
+// ... or per run of 4 input blocks (sp.in_group): 0 when not, else the number of slices its reduction over the tokens is
+// best split into (1: no split).  With more than one slice the caller sets p.ksplit = slices, p.split_stride = elements of the
+// weight gradient, and points epi.out at fp32 partial sums (lt_sparse_dw_split_workspace bytes) that it sums afterwards.
+int lt_sparse_dw_in_grouped_slices(const GemmProblem& p);
+size_t lt_sparse_dw_split_workspace(int64_t in_features, int blocks_per_in, int in_group, int64_t tokens);
 // whether the bf16 matrix-core walk for 64 x 64 blocks takes this block-sparse problem with epilogue `kind`
 bool lt_sparse_mfma_supported(const GemmProblem& p, int kind);
 int lt_launch_gemm_sparse(const GemmProblem& p, int kind, int dtype, int io_dtype, hipStream_t stream);

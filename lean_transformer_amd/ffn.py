@@ -246,7 +246,7 @@ class _LeanFFN(torch.autograd.Function):
                        None if fwd is None else fwd.to(torch.int32).contiguous(),
                        None if bwd is None else bwd.to(torch.int64).contiguous())
             keep.append(tensors)
-            projections.append(linear_desc(*tensors, index_owner=fwd))
+            projections.append(linear_desc(*tensors, index_owner=fwd, backward_owner=bwd))
         desc = nat.LtFfnDesc()
         desc.tokens, desc.hidden = tokens, hidden
         desc.intermediate = projections[1].in_features

@@ -288,6 +288,45 @@ def test_bf16_blocksparse_layers_with_and_without_shared_list_runs(tokens, fan_i
         assert_close(a, b, BF16, name)
 
 
+@pytest.mark.parametrize("tokens", [256, 300, 1024, 2048])
+@pytest.mark.parametrize("fan_in,fan_out,stretch,run", [(4096, 1024, True, 4), (4096, 512, True, 8), (4096, 1024, False, 1)])
+@pytest.mark.parametrize("lowrank_dim", [0, 64])
+def test_bf16_blocksparse_wide_layers_with_runs_on_the_input_side(tokens, fan_in, fan_out, stretch, run, lowrank_dim):
+    """PixelFly stretched over a wide matrix: the input blocks come in runs with one list of output blocks and the weight
+    gradient runs as dense products over gathered blocks of dY (2048 tokens: with its reduction over the tokens split in two;
+    300 tokens, not a multiple of 32: the walk); tiled, everything is a walk.  Against fp32 stock ops on the dense expansion
+    of the same weights."""
+    from lean_transformer_amd.blocksparse.linear import shared_input_run, shared_list_run
+    torch.manual_seed(tokens + fan_out + lowrank_dim)
+    layout = f"pixelfly(block_size=64, stretch={stretch})"
+    layer = lt.GeneralizedLinear(lt.GeneralizedMatrix(fan_in, fan_out, layout, lowrank_dim), bias=True)
+    with torch.no_grad():
+        layer.bias.normal_(std=0.1)
+        layer.weight.normal_(std=0.05)
+        if lowrank_dim:
+            layer.matrix.lowrank_first.normal_(std=0.05)
+            layer.matrix.lowrank_second.normal_(std=0.05)
+    layer = layer.to(DEV).to(BF16)
+    matrix = layer.matrix
+    assert shared_input_run(matrix.backward_indices) == run
+    assert shared_list_run(matrix.forward_indices, matrix.backward_indices.shape[1]) == 1
+    x, dy = torch.randn(tokens, fan_in), torch.randn(tokens, fan_out)
+    xd = x.to(DEV).to(BF16).requires_grad_(True)
+    y = layer(xd)
+    names, params = zip(*layer.named_parameters())
+    grads = torch.autograd.grad(y, [xd, *params], dy.to(DEV).to(BF16))
+    leaves = {n: p.detach().float().requires_grad_(True) for n, p in layer.named_parameters()}
+    xr = x.to(DEV).to(BF16).float().requires_grad_(True)
+    y_ref = xr @ _dense_from_native(leaves["matrix.weight"], matrix.backward_indices, fan_out).t() + leaves["bias"]
+    if lowrank_dim:
+        y_ref = y_ref + (xr @ leaves["matrix.lowrank_first"].t()) @ leaves["matrix.lowrank_second"].t()
+    ref = torch.autograd.grad(y_ref, [xr, *[leaves[n] for n in names]], dy.to(DEV).to(BF16).float())
+    assert_close(y, y_ref.detach(), BF16, "y")
+    assert_close(grads[0], ref[0], BF16, "dx")
+    for name, a, b in zip(names, grads[1:], ref[1:]):
+        assert_close(a, b, BF16, name)
+
+
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("tokens", [512, 300])
 def test_bf16_ffn_with_blocksparse_projections_in_runs(gated, tokens):

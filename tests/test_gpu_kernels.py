@@ -385,3 +385,56 @@ def test_out_group_promise_is_checked_on_the_device_and_a_false_one_stays_inside
     ref = obs.blocksparse_matmul(x.float().cpu(), sq.weight.detach().float().cpu(), sq.forward_indices.cpu().numpy())
     assert_close(outs[0], ref, torch.bfloat16, "y without the promise")
     assert not torch.equal(outs[0], outs[1])
+
+
+def test_in_group_promise_is_checked_on_the_device_and_a_false_one_stays_inside_the_gradient():
+    """lt_linear.in_group: the same promise on the input side (runs of input blocks with one list of output blocks).
+    lt_linear_check_in_group tests it on the device; a value that does not divide the number of input blocks is refused; a
+    false promise writes wrong values into the weight gradient, all of them inside it (a guard band behind it stays intact)."""
+    from lean_transformer_amd.blocksparse.linear import linear_desc
+    torch.manual_seed(4)
+    m = lt.GeneralizedMatrix(4096, 1024, "pixelfly(block_size=64, stretch=True)", 0).to(DEV).to(torch.bfloat16)
+    run = 4096 // 1024
+    fwd, bwd = m.forward_indices, m.backward_indices
+    lib = nat.lib()
+    flag = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    stream = nat.current_stream(flag.device)
+
+    def checked(group):
+        desc = linear_desc(m.weight.detach(), None, None, None, fwd, bwd)
+        desc.in_group = group
+        status = lib.lt_linear_check_in_group(desc, nat.ptr(flag), stream)
+        return status, (int(flag.item()) if status == 0 else None)
+
+    desc = linear_desc(m.weight.detach(), None, None, None, fwd, bwd)
+    assert desc.in_group == run and desc.out_group == 1
+    assert checked(run) == (0, 1) and checked(2) == (0, 1) and checked(1) == (0, 1) and checked(0) == (0, 1)
+    assert checked(8) == (0, 0) and checked(16) == (0, 0)
+    assert checked(3)[0] != 0 and "in_group" in lib.lt_last_error().decode()  # 64 input blocks are not a multiple of 3
+    # weight gradient with the true promise, without one, and with a false one (a square layout claimed to have runs of 4)
+    tokens = 1024
+    sq = lt.GeneralizedMatrix(2048, 2048, "pixelfly(block_size=64)", 0).to(DEV).to(torch.bfloat16)
+    grads_of = {}
+    for name, matrix, groups in (("wide", m, (0, run)), ("square", sq, (0, 4))):
+        in_f, out_f = matrix.weight.shape[0], matrix.forward_indices.shape[0] * 64
+        x = torch.randn(tokens, in_f, device=DEV).to(torch.bfloat16)
+        dy = torch.randn(tokens, out_f, device=DEV).to(torch.bfloat16)
+        for group in groups:
+            desc = linear_desc(matrix.weight.detach(), None, None, None, matrix.forward_indices, matrix.backward_indices)
+            desc.in_group = group
+            room = torch.full((matrix.weight.numel() + 65536,), 7.0, dtype=torch.bfloat16, device=DEV)
+            grads = nat.LtLinearGrads()
+            grads.weight = nat.ptr(room)
+            need = lib.lt_linear_backward_workspace_bytes(desc, tokens, nat.dtype_code(torch.bfloat16))
+            ws = torch.empty(max(int(need), 1), dtype=torch.uint8, device=DEV)
+            nat.check(lib.lt_linear_backward(desc, tokens, nat.dtype_code(torch.bfloat16), nat.ptr(x), nat.ptr(dy), None, None,
+                                             grads, nat.ptr(ws), ws.numel(), stream), "lt_linear_backward")
+            assert bool((room[matrix.weight.numel():] == 7.0).all()), (name, group)
+            assert torch.isfinite(room.float()).all()
+            grads_of[name, group] = room[:matrix.weight.numel()].clone()
+        ref = obs.blocksparse_matmul_backward(dy.float().cpu(), x.float().cpu(), matrix.weight.detach().float().cpu(),
+                                              matrix.backward_indices.cpu().numpy())[1]
+        assert_close(grads_of[name, 0].view_as(matrix.weight), ref, torch.bfloat16, name + " without the promise")
+    assert_close(grads_of["wide", run].view_as(m.weight), grads_of["wide", 0].float().view_as(m.weight), torch.bfloat16, "wide")
+    assert not torch.equal(grads_of["square", 0], grads_of["square", 4])
+

@@ -258,6 +258,21 @@ def test_native_and_block_list_weight_orders():
         lt.block_list_to_native(blocks, coords.flip(1), m.backward_indices[:, :1])
 
 
+def test_shared_input_run_of_pixelfly_layouts():
+    """runs of consecutive input blocks with one list of output blocks: stretched PixelFly on a wide matrix repeats every list
+    in_blocks / out_blocks times; tall, square and tiled layouts have none; the cached value follows in-place changes"""
+    from lean_transformer_amd.blocksparse.linear import shared_input_run
+    for out_f, in_f, stretch, expected in [(1024, 4096, True, 4), (512, 4096, True, 8), (1024, 4096, False, 1),
+                                           (1024, 1024, True, 1), (4096, 1024, True, 1)]:
+        layout = lt.get_blocksparse_layout(out_f, in_f, f"pixelfly(block_size=64, stretch={stretch})")
+        _, backward_indices = lt.get_indices_from_layout(layout)
+        assert shared_input_run(backward_indices) == expected, (out_f, in_f, stretch)
+    _, backward_indices = lt.get_indices_from_layout(lt.get_blocksparse_layout(1024, 4096, "pixelfly(block_size=64, stretch=True)"))
+    assert shared_input_run(backward_indices) == 4
+    backward_indices[1] = backward_indices[8]
+    assert shared_input_run(backward_indices) == 1
+
+
 def test_shared_list_run_of_pixelfly_layouts():
     """runs of consecutive output blocks with one list of input blocks: stretched PixelFly on a tall matrix repeats every list
     out_blocks / in_blocks times, the tiled form and square matrices have none; the cached value follows in-place changes"""
