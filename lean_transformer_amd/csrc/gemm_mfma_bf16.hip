@@ -181,7 +181,10 @@ int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* w
   int slices = 1;
   if (workspace && tiles < 192) {
     // two workgroups per CU (64 KiB of LDS each): the slices are short and bound by load latency
-    slices = (int)std::min<int64_t>(std::min<int64_t>(512 / tiles, kt_total / 4), SKINNY_MAX_SLICES);
+    // (one workgroup per CU where a slice's fp32 partial result is as large as the operand tile it read: with twice the
+    // slices the partial sums cost more than the second workgroup hides -- measured on [4096, 128] results)
+    const int64_t workgroups = tiles <= 64 ? 256 : 512;
+    slices = (int)std::min<int64_t>(std::min<int64_t>(workgroups / tiles, kt_total / 4), SKINNY_MAX_SLICES);
     const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.M * (size_t)p.N * sizeof(float)));
     slices = (int)std::max<int64_t>(1, std::min<int64_t>(slices, fit));
   }
