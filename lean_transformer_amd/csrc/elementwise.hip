@@ -338,13 +338,52 @@ __global__ __launch_bounds__(256) void colreduce4_kernel(int rows, int64_t strid
   }
 }
 
-// out[c] = sum of `rows` rows of partial: picks the vector kernel when the layout allows
-static void launch_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream) {
-  if ((cols & 3) == 0 && (stride & 3) == 0 && lt_aligned(partial, 16) && lt_aligned(out, 16))
+// several such sums in one launch: blockIdx.y picks the job; the same arithmetic in the same order as colreduce4_kernel
+__global__ __launch_bounds__(256) void colreduce4_multi_kernel(ColReduceQueue q) {
+  __shared__ float red[16][16][5];
+  const ColReduceJob& job = q.job[blockIdx.y];
+  const int cl = threadIdx.x & 15, rl = threadIdx.x >> 4;
+  const int c = (blockIdx.x * 16 + cl) * 4;
+  if (blockIdx.x * 64 >= job.cols) return;  // (the whole workgroup)
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < job.cols) {
+    for (int r = rl; r < job.rows; r += 16) {
+      float v[4];
+      load4(job.partial + (int64_t)r * job.stride + c, v);
+#pragma unroll
+      for (int e = 0; e < 4; e++) s[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) red[rl][cl][e] = s[e];
+  __syncthreads();
+  if (rl == 0 && c < job.cols) {
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      o[e] = 0.f;
+#pragma unroll
+      for (int k = 0; k < 16; k++) o[e] += red[k][cl][e];
+    }
+    store4(job.out + c, o);
+  }
+}
+
+// out[c] = sum of `rows` rows of partial: picks the vector kernel when the layout allows; with a queue that has room, the
+// vector form waits for the queue's flush
+static void launch_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream,
+                             ColReduceQueue* defer = nullptr) {
+  const bool vec = (cols & 3) == 0 && (stride & 3) == 0 && lt_aligned(partial, 16) && lt_aligned(out, 16);
+  if (vec && defer && defer->n < 4) {
+    defer->job[defer->n++] = ColReduceJob{partial, out, rows, cols, stride};
+    return;
+  }
+  if (vec)
     hipLaunchKernelGGL(colreduce4_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(256), 0, stream, rows, stride, cols, partial, out);
   else
     hipLaunchKernelGGL(colreduce_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, stream, rows, stride, cols, partial, out);
 }
+
 
 // partial[blockIdx.y][c] = sum over this row-slice of in[t, c]; 64 column lanes x 4 row lanes per workgroup
 template <typename T>
@@ -634,7 +673,7 @@ size_t lt_ln_backward_workspace(int64_t T, int H) {
 
 int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* stats, const float* w, int dy_dtype,
                    const void* dy, int dx_dtype, const void* residual_grad, void* dx, float* dweight, float* dbias,
-                   void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                   void* workspace, size_t workspace_bytes, hipStream_t stream, ColReduceQueue* defer) {
   LT_REQUIRE(T > 0 && H > 0 && x && stats && w && dy, LT_ERR_BAD_ARG, "layernorm backward: bad arguments");
   LT_REQUIRE(H <= 256 * LNB_MAXC, LT_ERR_UNSUPPORTED, "layernorm backward: hidden size %d above %d", H, 256 * LNB_MAXC);
   LT_REQUIRE((dweight == nullptr) == (dbias == nullptr), LT_ERR_BAD_ARG, "layernorm backward: pass both dweight and dbias or neither");
@@ -716,10 +755,8 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   }
   if (dweight) {
     // partial rows alternate (dweight, dbias): stride 2 * H between them
-    launch_colreduce(partial_rows, (int64_t)2 * H, H,
-                       partial, dweight, stream);
-    launch_colreduce(partial_rows, (int64_t)2 * H, H,
-                       partial + H, dbias, stream);
+    launch_colreduce(partial_rows, (int64_t)2 * H, H, partial, dweight, stream, defer);
+    launch_colreduce(partial_rows, (int64_t)2 * H, H, partial + H, dbias, stream, defer);
     LT_LAUNCH_CHECK();
   }
   return LT_OK;
@@ -880,7 +917,7 @@ int lt_dropout_cast(int64_t n, int in_dtype, const void* in, int out_dtype, void
 // lt_dropout_cast of a [rows, cols] tensor plus colsum[c] = sum over rows of the result; workspace as for lt_colsum
 int lt_dropout_cast_colsum(int64_t rows, int cols, int in_dtype, const void* in, int out_dtype, void* out,
                            const DropoutParams& drop, float* colsum, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream) {
+                           hipStream_t stream, ColReduceQueue* defer) {
   LT_REQUIRE(rows > 0 && cols > 0 && in && out && colsum, LT_ERR_BAD_ARG, "dropout + column sums: bad arguments");
   LT_REQUIRE(workspace && workspace_bytes >= lt_colsum_workspace(rows, cols), LT_ERR_WORKSPACE,
              "dropout + column sums: workspace of %zu bytes needed", lt_colsum_workspace(rows, cols));
@@ -901,7 +938,7 @@ int lt_dropout_cast_colsum(int64_t rows, int cols, int in_dtype, const void* in,
     case 2: hipLaunchKernelGGL((dropout_cast_colsum_kernel<bf16, float>), grid, block, 0, stream, rows, cols, (const bf16*)in, (float*)out, drop, rps, partial); break;
     default: hipLaunchKernelGGL((dropout_cast_colsum_kernel<bf16, bf16>), grid, block, 0, stream, rows, cols, (const bf16*)in, (bf16*)out, drop, rps, partial); break;
   }
-  launch_colreduce(slices, (int64_t)cols, cols, partial, colsum, stream);
+  launch_colreduce(slices, (int64_t)cols, cols, partial, colsum, stream, defer);
   LT_LAUNCH_CHECK();
   return LT_OK;
 }
@@ -927,8 +964,28 @@ int lt_splitk_reduce(const float* partial, int slices, int64_t stride, int64_t c
   return LT_OK;
 }
 
-int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream) {
+int lt_colreduce_flush(ColReduceQueue& queue, hipStream_t stream) {
+  if (queue.n == 0) return LT_OK;
+  int blocks = 1;
+  double bytes = 0.0;
+  for (int i = 0; i < queue.n; i++) {
+    blocks = std::max(blocks, (queue.job[i].cols + 63) / 64);
+    bytes += (double)queue.job[i].cols * 4.0 * (queue.job[i].rows + 1);
+  }
+  LtProfileScope scope("colreduce", 0.0, bytes, stream);
+  hipLaunchKernelGGL(colreduce4_multi_kernel, dim3((unsigned)blocks, (unsigned)queue.n), dim3(256), 0, stream, queue);
+  queue.n = 0;
+  LT_LAUNCH_CHECK();
+  return LT_OK;
+}
+
+int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream,
+                 ColReduceQueue* defer) {
   LT_REQUIRE(rows > 0 && cols > 0 && partial && out, LT_ERR_BAD_ARG, "colreduce: bad arguments");
+  if (defer && defer->n < 4 && (cols & 3) == 0 && (stride & 3) == 0 && lt_aligned(partial, 16) && lt_aligned(out, 16)) {
+    launch_colreduce(rows, stride, cols, partial, out, stream, defer);
+    return LT_OK;
+  }
   LtProfileScope scope("colreduce", 0.0, (double)cols * 4.0 * (rows + 1), stream);
   launch_colreduce(rows, stride, cols, partial, out, stream);
   LT_LAUNCH_CHECK();

@@ -495,6 +495,10 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   const int cdt = d.compute_dtype, io = d.io_dtype;
   const DropoutParams drop = make_dropout(d.dropout_p, d.dropout_seed, d.dropout_offset);
 
+  // the small column sums at the end of three passes (two bias gradients, the LayerNorm parameter gradients) wait for one
+  // launch at the end of the step
+  ColReduceQueue reduces;
+  reduces.n = 0;
   // gradient entering the down-projection: dropout replayed on dy, then (optionally) back through the post-LN
   const void* g = s.g;
   lt_linear_grads h2o_grads = grads->h2o;
@@ -503,7 +507,7 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   } else if (h2o_grads.bias && !d.post_ln_weight) {
     // the same pass also sums the columns of g: the down-projection's bias gradient
     LT_TRY(lt_dropout_cast_colsum(T, (int)H, io, dy, cdt, s.g, drop, (float*)h2o_grads.bias, s.h2o.colsum, s.h2o.colsum_bytes,
-                                  stream));
+                                  stream, &reduces));
     h2o_grads.bias = nullptr;
   } else {
     LT_TRY(lt_dropout_cast(T * H, io, dy, cdt, s.g, drop, stream));
@@ -528,7 +532,8 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   }
   lt_linear_grads i2h_grads = grads->i2h;
   if (bias_rows > 0) {  // db1 = column sums of dP, already reduced to one row per bias_rows tokens
-    LT_TRY(lt_colreduce((int)((T + bias_rows - 1) / bias_rows), N1, (int)N1, s.act_colsum, (float*)grads->i2h.bias, stream));
+    LT_TRY(lt_colreduce((int)((T + bias_rows - 1) / bias_rows), N1, (int)N1, s.act_colsum, (float*)grads->i2h.bias, stream,
+                        &reduces));
     i2h_grads.bias = nullptr;
   }
 
@@ -543,9 +548,9 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
   }
   if (need_du) {
     LT_TRY(lt_ln_backward(T, (int)H, io, x, saved->ln_stats, d.ln_weight, LT_F32, s.du, io, d.residual ? dy : nullptr,
-                          grads->dx, grads->ln_weight, grads->ln_bias, s.ln_ws, s.ln_ws_bytes, stream));
+                          grads->dx, grads->ln_weight, grads->ln_bias, s.ln_ws, s.ln_ws_bytes, stream, &reduces));
   }
-  return LT_OK;
+  return lt_colreduce_flush(reduces, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------

@@ -498,8 +498,23 @@ size_t lt_gemm_generic_splitk_workspace(int64_t M, int64_t N, int64_t K);
 // rows per partial row of EpiParams::colsum when lt_launch_gemm / lt_launch_gemm_sparse sends this EPI_ACT_BWD problem to a
 // kernel that fills it (128: copy-based dense kernel; 64: block-sparse walk on whole tiles with the tanh GELU); 0: it will not
 int lt_gemm_colsum_rows(const GemmProblem& p, int dtype, int io_dtype);
-// out[c] = sum over `rows` partial rows of partial[r * stride + c]
-int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream);
+// Column sums of partial rows that may wait: a caller that runs several passes with such a tail (the FFN backward: two bias
+// gradients and the LayerNorm parameter gradients) hands the same queue to each of them and flushes it once, one launch
+// for all sums instead of one each.  The partial rows must stay untouched until the flush.
+struct ColReduceJob {
+  const float* partial;
+  float* out;
+  int rows, cols;
+  int64_t stride;
+};
+struct ColReduceQueue {
+  ColReduceJob job[4];
+  int n;
+};
+int lt_colreduce_flush(ColReduceQueue& queue, hipStream_t stream);
+// out[c] = sum over `rows` partial rows of partial[r * stride + c] (now, or at the flush of `defer`)
+int lt_colreduce(int rows, int64_t stride, int cols, const float* partial, float* out, hipStream_t stream,
+                 ColReduceQueue* defer = nullptr);
 int lt_launch_gemm_skinny(const GemmProblem& p, int dtype, int io_dtype, void* workspace, size_t workspace_bytes,
                           hipStream_t stream);
 // EPI_OUT problems with few output tiles and a long reduction (the down-projection of a short batch): the reduction split
