@@ -8,8 +8,9 @@ K steps are timed by wall clock; the same K steps are then repeated with a HIP e
 (recorded by the library on the launch stream) and `roofline` is computed from the GEMM launches of that pass;
 `cpu_baseline` times the CPU oracle (tests' checker, not the product) on a bounded sample of the same workload.
 The default run also measures configurations 2 and 4 (about a second of GPU time each) and reports them under
-`extra_configs` of the same line; `--config c5` times the full GPT train step of configuration 5 (the stock-PyTorch model of
-tests/gpt_harness.py around the FFN kernels).
+`extra_configs` of the same line; `--config c4t` is configuration 4 with the reference's default layout (stretch=False);
+`--config c5` times the full GPT train step of configuration 5 (the stock-PyTorch model of tests/gpt_harness.py around the
+FFN kernels).
 """
 import argparse
 import hashlib
@@ -39,6 +40,12 @@ CONFIGS = {
     "c4": dict(batch=2, seq=2048, hidden=4096, inter=16384, gated=True, std=0.02, dropout=0.0, dtype="bf16", sparse=True,
                name="config4: LeanFFN PixelFly (64x64 blocks, stretch, density 7/64) + rank-128 low-rank GeGLU fwd+bwd, "
                     "hidden 4096, intermediate 16384, x [2,2048,4096], bf16"),
+    # config 4 with the reference's default layout (pixelfly tiles the square butterfly instead of stretching it: no runs of
+    # blocks with one list, every product is a walk over the index tables)
+    "c4t": dict(batch=2, seq=2048, hidden=4096, inter=16384, gated=True, std=0.02, dropout=0.0, dtype="bf16", sparse=True,
+                stretch=False,
+                name="config4, default layout: LeanFFN PixelFly (64x64 blocks, stretch=False, density 7/64) + rank-128 "
+                     "low-rank GeGLU fwd+bwd, hidden 4096, intermediate 16384, x [2,2048,4096], bf16"),
 }
 
 
@@ -48,7 +55,7 @@ def build_workload(torch, lt, cfg, device):
     n1 = 2 * inter if cfg["gated"] else inter
     x = torch.randn(cfg["batch"], cfg["seq"], hidden, generator=g)
     if cfg["sparse"]:
-        layout = "pixelfly(block_size=64, stretch=True)"
+        layout = f"pixelfly(block_size=64, stretch={cfg.get('stretch', True)})"
         up = lt.GeneralizedLinear(lt.GeneralizedMatrix(hidden, n1, layout, 128))
         down = lt.GeneralizedLinear(lt.GeneralizedMatrix(inter, hidden, layout, 128))
         ffn = lt.LeanFFN(hidden, inter, gated=cfg["gated"], layer_norm_eps=1e-5, dropout=cfg["dropout"], i2h_proj=up,
@@ -162,11 +169,14 @@ def measured_traffic(config):
     configuration (written when that summary is refreshed), with the algorithmic bytes of the same launches and where the
     figure comes from: the summary records the hash of the kernel sources it was measured on, and `stale` says whether the
     tree's kernels still are those.  (None, None, None) when the configuration has no such summary."""
-    path = os.path.join(ROOT, "profiles", f"leanffn_config{config[1:]}_gemm_hbm_traffic.json")
+    counted = config != "c4t"  # the default-layout variant of config 4 has config 4's algorithmic bytes and no counter run
+    path = os.path.join(ROOT, "profiles", f"leanffn_config{config[1:2]}_gemm_hbm_traffic.json")
     if not os.path.exists(path):
         return None, None, None
     with open(path) as f:
         d = json.load(f)
+    if not counted:
+        return None, float(d["algorithmic_bytes_per_gemm_launch"]), None
     tree = csrc_sha16()
     source = {"file": os.path.relpath(path, ROOT), "measured_on_csrc_sha16": d.get("csrc_sha16"), "tree_csrc_sha16": tree,
               "stale": d.get("csrc_sha16") != tree}
@@ -313,7 +323,7 @@ def summarise(run, config_name):
                 "kernel": "all GEMM launches of a step: " + ", ".join(sorted({k[0] for k in gemm})),
                 "flops_per_launch": gemm_flops / max(gemm_launches, 1),
                 "avg_launch_us": gemm_ms / max(gemm_launches, 1) * 1e3}
-    if cfg["sparse"] and traffic:
+    if cfg["sparse"] and traffic_algorithmic:
         # The block-sparse configuration is bound by memory traffic (its GEMM launches move 5 TB/s through the L2 boundary with
         # the matrix cores a quarter busy): priced against HBM with the launches' algorithmic bytes (every operand and result
         # once, from the same counter summary) over their measured duration.
