@@ -83,13 +83,18 @@ typedef struct lt_linear {
                              in_blocks.  A promise by the caller that only selects faster forward and weight-gradient
                              kernels; 0 or 1 when not known, which is always safe.  Must divide the number of output blocks.
                              A false promise computes with the wrong weight blocks (it cannot make a kernel read outside
-                             the weight); lt_linear_check_out_group tests it on the device. */
+                             the weight); lt_linear_check_out_group tests it on the device.
+                             Low 16 bits: the run length.  High 16 bits, when above 1: the members of a run are not
+                             consecutive but that many blocks apart (blocks r, r + s, r + 2 s, ...: PixelFly with stretch=False
+                             on a tall matrix tiles a square pattern s blocks wide; length x s must equal the number of
+                             output blocks).  Such a run promises equal lists of input blocks only and serves the
+                             weight-gradient kernel only. */
   int32_t in_group;       /* sparse: every aligned run of this many consecutive input blocks has the same list of output
                              blocks (backward_indices of input block ib0 + i = those of ib0).  PixelFly with stretch=True on
                              a wide matrix: in_blocks / out_blocks.  A promise like out_group: it only selects a faster
                              weight-gradient kernel, 0 or 1 is always safe, it must divide the number of input blocks, a false
                              one puts wrong values into the weight gradient (never an access outside it), and
-                             lt_linear_check_in_group tests it on the device. */
+                             lt_linear_check_in_group tests it on the device.  Low / high 16 bits as in out_group. */
 } lt_linear;
 
 /* Where lt_linear_backward / lt_ffn_backward write parameter gradients; a NULL member skips that gradient.

@@ -164,6 +164,52 @@ def shared_list_run(forward_indices: torch.Tensor, blocks_per_in: int) -> int:
     return run
 
 
+def _strided_run(lists: torch.Tensor) -> Tuple[int, int]:
+    """(g, s): the most members g (a power of two, g * s = number of blocks) such that blocks r, r + s, r + 2 s, ... all have the
+    same row in `lists` -- what tiling a square pattern s blocks wide g times gives; (1, 1) when there is no such structure"""
+    n = lists.shape[0]
+    g = 1
+    while n % (2 * g) == 0:
+        g *= 2
+    while g >= 2:
+        tiled = lists.reshape(g, n // g, -1)
+        if bool((tiled == tiled[:1]).all()):
+            return g, n // g
+        g //= 2
+    return 1, 1
+
+
+def shared_list_group(forward_indices: torch.Tensor, blocks_per_in: int) -> int:
+    """lt_linear.out_group of a layer with these index tables: the run of consecutive output blocks with one list of input
+    blocks (shared_list_run) when that is 4 or more; else, when output blocks a fixed number of blocks apart share their lists
+    (PixelFly with ``stretch=False`` on a tall matrix tiles the square butterfly), the number of such blocks in the low 16
+    bits and their distance in the high 16 bits; else the run (1 ... 2).  Remembered on the tensor like shared_list_run."""
+    run = shared_list_run(forward_indices, blocks_per_in)
+    if run >= 4:
+        return run
+    cached = getattr(forward_indices, "_lt_shared_list_group", None)
+    if cached is not None and cached[0] == (forward_indices._version, blocks_per_in):
+        return cached[1]
+    members, stride = _strided_run(torch.div(forward_indices, blocks_per_in, rounding_mode="floor"))
+    group = (members | (stride << 16)) if (members >= 4 and 1 < stride < 1 << 15 and members < 1 << 16) else run
+    forward_indices._lt_shared_list_group = ((forward_indices._version, blocks_per_in), group)
+    return group
+
+
+def shared_input_group(backward_indices: torch.Tensor) -> int:
+    """lt_linear.in_group: the same on the input side (shared_input_run, else blocks a fixed distance apart)"""
+    run = shared_input_run(backward_indices)
+    if run >= 4:
+        return run
+    cached = getattr(backward_indices, "_lt_shared_input_group", None)
+    if cached is not None and cached[0] == backward_indices._version:
+        return cached[1]
+    members, stride = _strided_run(backward_indices)
+    group = (members | (stride << 16)) if (members >= 4 and 1 < stride < 1 << 15 and members < 1 << 16) else run
+    backward_indices._lt_shared_input_group = (backward_indices._version, group)
+    return group
+
+
 def shared_input_run(backward_indices: torch.Tensor) -> int:
     """The same on the input side: the largest power of two g such that every aligned run of g consecutive input blocks has
     the same list of output blocks (PixelFly with ``stretch=True`` on a matrix with more input than output blocks: ``in_blocks
@@ -201,11 +247,9 @@ def linear_desc(weight, bias_f32, lowrank_first, lowrank_second, forward_indices
         desc.block, desc.blocks_per_in, desc.blocks_per_out = block, blocks_per_in, forward_indices.shape[1]
         desc.forward_indices, desc.backward_indices = nat.ptr(forward_indices), nat.ptr(backward_indices)
         owner = forward_indices if index_owner is None else index_owner
-        desc.out_group = shared_list_run(owner, blocks_per_in)
-        if desc.out_group > 1 and forward_indices.shape[0] % desc.out_group:
-            desc.out_group = 1  # (cannot happen for a power of two that divides the block count; the C ABI refuses it)
+        desc.out_group = shared_list_group(owner, blocks_per_in)
         if backward_indices is not None:
-            desc.in_group = shared_input_run(backward_indices if backward_owner is None else backward_owner)
+            desc.in_group = shared_input_group(backward_indices if backward_owner is None else backward_owner)
     return desc
 
 

@@ -49,6 +49,9 @@ int check_dtype(int d, const char* what) {
 
 // which index tables a call reads: the forward walk takes forward_indices, both gradient walks take backward_indices
 enum { NEED_FWD_TABLE = 1, NEED_BWD_TABLE = 2 };
+// lt_linear::out_group / in_group: run length in the low 16 bits, blocks between the members of a run in the high 16 bits
+inline int group_length(int32_t g) { return g & 0xffff; }
+inline int group_stride(int32_t g) { return (g >> 16) & 0x7fff; }
 
 int check_linear(const lt_linear& lin, const char* name, int tables = NEED_FWD_TABLE | NEED_BWD_TABLE) {
   LT_REQUIRE(lin.weight && lin.in_features > 0 && lin.out_features > 0, LT_ERR_BAD_ARG, "%s: weight / sizes missing", name);
@@ -64,10 +67,13 @@ int check_linear(const lt_linear& lin, const char* name, int tables = NEED_FWD_T
                    (int64_t)lin.blocks_per_in * (lin.in_features / lin.block) ==
                        (int64_t)lin.blocks_per_out * (lin.out_features / lin.block),
                LT_ERR_BAD_ARG, "%s: unbalanced layout (K=%d, A=%d)", name, lin.blocks_per_out, lin.blocks_per_in);
-    LT_REQUIRE(lin.out_group >= 0 && (lin.out_group <= 1 || (lin.out_features / lin.block) % lin.out_group == 0), LT_ERR_BAD_ARG,
-               "%s: out_group=%d does not divide the %d output blocks", name, lin.out_group, lin.out_features / lin.block);
-    LT_REQUIRE(lin.in_group >= 0 && (lin.in_group <= 1 || (lin.in_features / lin.block) % lin.in_group == 0), LT_ERR_BAD_ARG,
-               "%s: in_group=%d does not divide the %d input blocks", name, lin.in_group, lin.in_features / lin.block);
+    const int out_blocks = lin.out_features / lin.block, in_blocks = lin.in_features / lin.block;
+    const int og = group_length(lin.out_group), os = group_stride(lin.out_group);
+    const int ig = group_length(lin.in_group), is = group_stride(lin.in_group);
+    LT_REQUIRE(lin.out_group >= 0 && (og <= 1 || out_blocks % og == 0) && (os <= 1 || og * os == out_blocks), LT_ERR_BAD_ARG,
+               "%s: out_group (runs of %d, %d apart) does not fit the %d output blocks", name, og, os > 1 ? os : 1, out_blocks);
+    LT_REQUIRE(lin.in_group >= 0 && (ig <= 1 || in_blocks % ig == 0) && (is <= 1 || ig * is == in_blocks), LT_ERR_BAD_ARG,
+               "%s: in_group (runs of %d, %d apart) does not fit the %d input blocks", name, ig, is > 1 ? is : 1, in_blocks);
   }
   return LT_OK;
 }
@@ -75,20 +81,21 @@ int check_linear(const lt_linear& lin, const char* name, int tables = NEED_FWD_T
 namespace {
 // flag[0] = 0 when output block ob's list differs from that of the first block of its aligned run of `group`, or its weight
 // blocks do not follow that block's by ob % group (what lt_linear::out_group promises); untouched otherwise
+// (runs `stride` blocks apart promise the same lists of input blocks only: first block of the run = ob % stride)
 __global__ void check_out_group_kernel(const int32_t* __restrict__ forward_indices, int out_blocks, int per_out, int per_in,
-                                       int group, int32_t* flag) {
+                                       int group, int stride, int32_t* flag) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= out_blocks * per_out) return;
-  const int ob = i / per_out, e = i % per_out, ob0 = ob - ob % group;
+  const int ob = i / per_out, e = i % per_out, ob0 = stride > 1 ? ob % stride : ob - ob % group;
   const int mine = forward_indices[i], first = forward_indices[ob0 * per_out + e];
-  if (mine / per_in != first / per_in || mine != first + (ob - ob0)) flag[0] = 0;
+  if (mine / per_in != first / per_in || (stride <= 1 && mine != first + (ob - ob0))) flag[0] = 0;
 }
 // the same for lt_linear::in_group: input block ib's list of output blocks against that of the first block of its run
 __global__ void check_in_group_kernel(const int64_t* __restrict__ backward_indices, int in_blocks, int per_in, int group,
-                                      int32_t* flag) {
+                                      int stride, int32_t* flag) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= in_blocks * per_in) return;
-  const int ib = i / per_in, e = i % per_in, ib0 = ib - ib % group;
+  const int ib = i / per_in, e = i % per_in, ib0 = stride > 1 ? ib % stride : ib - ib % group;
   if (backward_indices[i] != backward_indices[ib0 * per_in + e]) flag[0] = 0;
 }
 __global__ void set_flag_kernel(int32_t* flag, int32_t value) { flag[0] = value; }
@@ -100,10 +107,11 @@ extern "C" int lt_linear_check_out_group(const lt_linear* lin, int32_t* flag, vo
   hipStream_t stream = (hipStream_t)stream_;
   hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, stream, flag, 1);
   LT_LAUNCH_CHECK();
-  if (lin->block > 0 && lin->out_group > 1) {
+  if (lin->block > 0 && group_length(lin->out_group) > 1) {
     const int out_blocks = lin->out_features / lin->block, entries = out_blocks * lin->blocks_per_out;
     hipLaunchKernelGGL(check_out_group_kernel, dim3((unsigned)((entries + 255) / 256)), dim3(256), 0, stream,
-                       lin->forward_indices, out_blocks, lin->blocks_per_out, lin->blocks_per_in, lin->out_group, flag);
+                       lin->forward_indices, out_blocks, lin->blocks_per_out, lin->blocks_per_in, group_length(lin->out_group),
+                       group_stride(lin->out_group), flag);
     LT_LAUNCH_CHECK();
   }
   return LT_OK;
@@ -115,10 +123,11 @@ extern "C" int lt_linear_check_in_group(const lt_linear* lin, int32_t* flag, voi
   hipStream_t stream = (hipStream_t)stream_;
   hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, stream, flag, 1);
   LT_LAUNCH_CHECK();
-  if (lin->block > 0 && lin->in_group > 1) {
+  if (lin->block > 0 && group_length(lin->in_group) > 1) {
     const int in_blocks = lin->in_features / lin->block, entries = in_blocks * lin->blocks_per_in;
     hipLaunchKernelGGL(check_in_group_kernel, dim3((unsigned)((entries + 255) / 256)), dim3(256), 0, stream,
-                       lin->backward_indices, in_blocks, lin->blocks_per_in, lin->in_group, flag);
+                       lin->backward_indices, in_blocks, lin->blocks_per_in, group_length(lin->in_group),
+                       group_stride(lin->in_group), flag);
     LT_LAUNCH_CHECK();
   }
   return LT_OK;
@@ -188,7 +197,7 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
   p.sp.mode = SPARSE_FWD; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
   p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
   p.sp.backward_indices = lin.backward_indices; p.sp.act = x; p.sp.ld_act = in; p.sp.weight = lin.weight;
-  p.sp.out_group = lin.out_group;
+  p.sp.out_group = group_length(lin.out_group); p.sp.out_stride = group_stride(lin.out_group);
   p.sp.walk_run = walk_run_for(lin.in_features / lin.block, lin.out_features / lin.block, lin.blocks_per_out);
   bool two_passes = gated && !(dtype == LT_BF16 && lt_sparse_mfma_supported(p, kind));
   if (gated && !two_passes) {
@@ -229,7 +238,8 @@ void plan_linear_backward(const lt_linear& lin, int64_t T, int dtype, Bump& ws, 
       s.skinny_bytes = std::max(s.skinny_bytes, lt_gemm_generic_splitk_workspace(T, lin.in_features, lin.out_features));
   }
   if (lin.block == 64 && dtype == LT_BF16)
-    s.skinny_bytes = std::max(s.skinny_bytes, lt_sparse_dw_split_workspace(lin.in_features, lin.blocks_per_in, lin.in_group, T));
+    s.skinny_bytes = std::max(s.skinny_bytes,
+                              lt_sparse_dw_split_workspace(lin.in_features, lin.blocks_per_in, group_length(lin.in_group), T));
   s.skinny = s.skinny_bytes ? ws.take(s.skinny_bytes) : nullptr;
 }
 
@@ -296,8 +306,9 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.act2 = x_act;
       p.sp.ld_act2 = in; p.sp.tokens = T;
-      p.sp.out_group = lin.forward_indices ? lin.out_group : 0;  // the grouped kernel reads the list from the forward table
-      p.sp.in_group = lin.in_group;
+      // (the grouped kernel reads the list from the forward table)
+      p.sp.out_group = lin.forward_indices ? group_length(lin.out_group) : 0; p.sp.out_stride = group_stride(lin.out_group);
+      p.sp.in_group = group_length(lin.in_group); p.sp.in_stride = group_stride(lin.in_group);
       p.epi = epi_store_params(grads.weight, lin.block, dtype, nullptr);
       const int slices = dtype == LT_BF16 ? lt_sparse_dw_in_grouped_slices(p) : 0;
       const size_t elements = (size_t)(in / lin.block) * lin.blocks_per_in * lin.block * lin.block;

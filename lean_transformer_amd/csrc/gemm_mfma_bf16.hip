@@ -299,7 +299,7 @@ bool lt_sparse_forward_grouped(const GemmProblem& p, int kind) {
   const SparseWalk& sp = p.sp;
   if (sp.mode != SPARSE_FWD || (kind != EPI_STORE && kind != EPI_ACT_FWD) || (kind == EPI_ACT_FWD && p.epi.gated)) return false;
   if (!lt_sparse_mfma_supported(p, kind)) return false;
-  if (sp.out_group < 4 || sp.out_group % 4 != 0 || p.N % 256 != 0) return false;
+  if (sp.out_group < 4 || sp.out_group % 4 != 0 || sp.out_stride > 1 || p.N % 256 != 0) return false;
   // the list travels in one register: at most 64 entries, input block and flat position in 16 bits each
   if (sp.blocks_per_out > 64 || sp.ld_act / 64 * sp.blocks_per_in > 65535) return false;
   if (p.nseg > 1 && p.K[1] % 64 != 0) return false;
@@ -312,6 +312,7 @@ bool lt_sparse_forward_grouped(const GemmProblem& p, int kind) {
 bool lt_sparse_dw_out_grouped(const GemmProblem& p) {
   const SparseWalk& sp = p.sp;
   const int64_t out_features = sp.ld_act;
+  if (sp.out_stride > 1 && (int64_t)sp.out_group * sp.out_stride * 64 != out_features) return false;  // runs must tile the blocks
   return sp.mode == SPARSE_DW && sp.out_group >= 4 && sp.out_group % 4 == 0 && sp.forward_indices && out_features % 256 == 0 &&
          sp.tokens % DK == 0 && sp.tokens > 0 && 32 * sp.ld_act * 2 + out_features * 2 < (int64_t)1 << 32 &&
          32 * sp.ld_act2 * 2 + p.N * 2 < (int64_t)1 << 32;
@@ -322,6 +323,7 @@ int lt_sparse_dw_in_grouped_slices(const GemmProblem& p) {
   const int64_t out_features = sp.ld_act, in_features = p.N;
   if (sp.mode != SPARSE_DW || !lt_sparse_mfma_supported(p, EPI_STORE) || lt_sparse_dw_out_grouped(p)) return 0;
   if (sp.in_group < 4 || sp.in_group % 4 != 0 || !sp.backward_indices || in_features % 256 != 0) return 0;
+  if (sp.in_stride > 1 && (int64_t)sp.in_group * sp.in_stride * 64 != in_features) return 0;  // runs must tile the blocks
   if (sp.tokens <= 0 || sp.tokens % DK != 0) return 0;
   if (32 * sp.ld_act * 2 + out_features * 2 >= (int64_t)1 << 32 || 32 * sp.ld_act2 * 2 + in_features * 2 >= (int64_t)1 << 32) return 0;
   // enough workgroups for the 256 CUs, each slice at least 32 k-steps long

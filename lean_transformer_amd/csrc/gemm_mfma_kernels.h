@@ -802,6 +802,16 @@ static_assert(copies_in_flight(false, false, {}, {}, false, 0) == 16 && copies_i
 constexpr BlockSlots SLOTS_NT_A = {{0, 0}}, SLOTS_NT_B = {{2, 2}}, SLOTS_NN_A = {{0, 2}};
 constexpr bool SPLIT_MN_B = true;
 
+// Block number of member j (0 .. 3) of the quad of run members that tile index t stands for.  Runs of `len` blocks that share
+// one list are either consecutive (stride 0 or 1: tile t is blocks 4 t .. 4 t + 3) or `stride` blocks apart (a layout tiled
+// from a square pattern `stride` blocks wide: run r is blocks r, r + stride, ...; tile t is quad t % (len / 4) of run
+// t / (len / 4)).
+__device__ __forceinline__ int lt_run_member(int t, int j, int len, int stride) {
+  if (stride <= 1) return t * 4 + j;
+  const int quads = len >> 2;
+  return t / quads + stride * ((t % quads) * 4 + j);
+}
+
 // Epilogue of one wavefront's (FM * 32) x 128 sub-tile of a copy-based kernel: acc[i][j] is the 32 x 32 block at rows
 // m0 + wm * WTM + 32 i, columns n0 + wn * 128 + 32 j of the result (gated forward: blocks 0, 1 gate columns, 2, 3 the
 // matching linear columns).  `stage` is 16 KiB of LDS that belongs to this wavefront alone; tile_rows x tile_cols is the
@@ -996,13 +1006,13 @@ __device__ __forceinline__ void dma_tile_epilogue(f32x16 (&acc)[FM][4], const Ge
     int64_t flat;
     if constexpr (SCATTER == 1) {
       per_out = p.sp.blocks_per_out;
-      const int64_t ob = m0 / 64 + (wm * WTM + i * 32) / 64;
+      const int64_t ob = lt_run_member((int)(m0 / 256), (wm * WTM + i * 32) / 64, p.sp.out_group, p.sp.out_stride);
       entry = (int)(n0 / 64) + wn * 2 + (c >> 6);
       flat = p.sp.forward_indices[ob * per_out + min(entry, per_out - 1)];
     } else {
       per_out = p.sp.blocks_per_in;
       entry = (int)(m0 / 64) + (wm * WTM + i * 32) / 64;
-      const int64_t ib = n0 / 64 + wn * 2 + (c >> 6);
+      const int64_t ib = lt_run_member((int)(n0 / 256), wn * 2 + (c >> 6), p.sp.in_group, p.sp.in_stride);
       flat = ib * per_out + min(entry, per_out - 1);
     }
     TO* dst = reinterpret_cast<TO*>(epi.out) + flat * 4096 + ((i & 1) * 32 + lane / LANES_PER_ROW) * 64 + (c & 63);
@@ -1234,15 +1244,24 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
       const GemmOperand x = {p.sp.act, p.sp.ld_act, 1};
       ca.setup(x, 0, m0, p.M, 0, wave, lane);  // unit u = column block u of X
     } else if constexpr (GATHER == 3) {
-      // the output blocks of list entries tm * 4 .. tm * 4 + 3 of input block tn * 4 (past the end: the last entry again)
+      // the output blocks of list entries tm * 4 .. tm * 4 + 3 of the first input block of tile column tn (past the end: the
+      // last entry again)
+      const int64_t ib0 = lt_run_member(tn, 0, p.sp.in_group, p.sp.in_stride);
       int blocks[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const int entry = min(tm * 4 + j, p.sp.blocks_per_in - 1);
-        blocks[j] = (int)p.sp.backward_indices[(int64_t)tn * 4 * p.sp.blocks_per_in + entry];
+        blocks[j] = (int)p.sp.backward_indices[ib0 * p.sp.blocks_per_in + entry];
       }
       const GemmOperand a = {p.A[0].ptr, p.A[0].ld, p.A[0].kmajor};
       ca.setup_gather(a, blocks, wave, lane);
+    } else if (GATHER == 1 && p.sp.out_stride > 1) {
+      // the four members of the run that tile row tm stands for lie out_stride blocks apart
+      int blocks[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) blocks[j] = lt_run_member(tm, j, p.sp.out_group, p.sp.out_stride);
+      const GemmOperand a = {p.A[0].ptr, p.A[0].ld, p.A[0].kmajor};
+      if constexpr (!A_KM) ca.setup_gather(a, blocks, wave, lane);
     } else {
       const GemmOperand a = {p.A[seg].ptr, p.A[seg].ld, p.A[seg].kmajor};
       ca.setup(a, seg, m0, p.M, 0, wave, lane);
@@ -1256,15 +1275,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
       return;
     }
     if constexpr (GATHER == 1) {
-      // the input blocks of list entries tn * 4 .. tn * 4 + 3 of output block tm * 4 (past the end: the last entry again)
+      // the input blocks of list entries tn * 4 .. tn * 4 + 3 of the first output block of tile row tm (past the end: the last
+      // entry again)
+      const int64_t ob0 = lt_run_member(tm, 0, p.sp.out_group, p.sp.out_stride);
       int blocks[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const int entry = min(tn * 4 + j, p.sp.blocks_per_out - 1);
-        blocks[j] = p.sp.forward_indices[(int64_t)tm * 4 * p.sp.blocks_per_out + entry] / p.sp.blocks_per_in;
+        blocks[j] = p.sp.forward_indices[ob0 * p.sp.blocks_per_out + entry] / p.sp.blocks_per_in;
       }
       const GemmOperand b = {p.B[0].ptr, p.B[0].ld, p.B[0].kmajor};
       cb.setup_gather(b, blocks, wave, lane);
+    } else if (GATHER == 3 && p.sp.in_stride > 1) {
+      int blocks[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) blocks[j] = lt_run_member(tn, j, p.sp.in_group, p.sp.in_stride);
+      const GemmOperand b = {p.B[0].ptr, p.B[0].ld, p.B[0].kmajor};
+      if constexpr (!B_KM) cb.setup_gather(b, blocks, wave, lane);
     } else {
       const GemmOperand b = {p.B[seg].ptr, p.B[seg].ld, p.B[seg].kmajor};
       cb.setup(b, seg, n0, p.N, (B_KM && gated) ? p.N : 0, wave, lane);

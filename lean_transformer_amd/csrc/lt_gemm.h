@@ -71,6 +71,10 @@ struct SparseWalk {
   // runs of 4 or more, and none on the output side, the weight gradient runs on 256 x 256 tiles of 4 list entries x 4 input
   // blocks.
   int in_group;
+  // blocks between the members of such a run: 0 or 1 = consecutive blocks; s > 1 = blocks r, r + s, r + 2 s, ... (a layout tiled
+  // from a square pattern s blocks wide; the group length times s is then the number of blocks).  Strided runs serve the
+  // weight gradient only.
+  int out_stride, in_stride;
   // FWD / DX walks (matrix-core kernel): order in which a group's index list is walked.  0 / 1: as listed.  g > 1 (must divide
   // the list's length n): entry (t % (n / g)) * g + t / (n / g) at step t, i.e. the first members of the list's runs of g,
   // then the second members, ...  In a stretched butterfly a list is made of runs of g consecutive blocks and the groups that

@@ -438,3 +438,27 @@ def test_in_group_promise_is_checked_on_the_device_and_a_false_one_stays_inside_
     assert_close(grads_of["wide", run].view_as(m.weight), grads_of["wide", 0].float().view_as(m.weight), torch.bfloat16, "wide")
     assert not torch.equal(grads_of["square", 0], grads_of["square", 4])
 
+
+def test_strided_run_promises_of_tiled_layouts_are_checked_on_the_device():
+    """tiled PixelFly layouts: the runs are blocks a square width apart; the check entries accept the true (length, distance)
+    pair, raise the flag's 0 for a wrong distance, and refuse a pair that does not tile the blocks"""
+    from lean_transformer_amd.blocksparse.linear import linear_desc
+    lib = nat.lib()
+    flag = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    stream = nat.current_stream(flag.device)
+    tall = lt.GeneralizedMatrix(1024, 4096, "pixelfly(block_size=64, stretch=False)", 0).to(DEV).to(torch.bfloat16)
+    wide = lt.GeneralizedMatrix(4096, 1024, "pixelfly(block_size=64, stretch=False)", 0).to(DEV).to(torch.bfloat16)
+    for m, field, entry in ((tall, "out_group", lib.lt_linear_check_out_group), (wide, "in_group", lib.lt_linear_check_in_group)):
+        desc = linear_desc(m.weight.detach(), None, None, None, m.forward_indices, m.backward_indices)
+        assert getattr(desc, field) == 4 | (16 << 16)
+
+        def checked(value):
+            setattr(desc, field, value)
+            status = entry(desc, nat.ptr(flag), stream)
+            return status, (int(flag.item()) if status == 0 else None)
+
+        assert checked(4 | (16 << 16)) == (0, 1)
+        assert checked(2 | (32 << 16)) == (0, 1)   # (blocks two square widths apart share their lists too)
+        assert checked(8 | (8 << 16)) == (0, 0)    # blocks half a square width apart do not
+        assert checked(4 | (8 << 16))[0] != 0      # 4 x 8 is not the 64 blocks
+

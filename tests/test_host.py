@@ -273,6 +273,20 @@ def test_shared_input_run_of_pixelfly_layouts():
     assert shared_input_run(backward_indices) == 1
 
 
+def test_strided_runs_of_tiled_pixelfly_layouts():
+    """PixelFly with stretch=False tiles the square butterfly: blocks one square width apart share their lists.  The group
+    value for the C ABI carries the number of such blocks in its low 16 bits and their distance in the high 16 bits; stretched
+    layouts keep their plain run length; square ones have neither"""
+    from lean_transformer_amd.blocksparse.linear import shared_input_group, shared_list_group
+    for out_f, in_f, stretch, out_group, in_group in [
+            (4096, 1024, False, 4 | (16 << 16), 1), (1024, 4096, False, 1, 4 | (16 << 16)), (4096, 512, False, 8 | (8 << 16), 1),
+            (4096, 1024, True, 4, 1), (1024, 4096, True, 1, 4), (1024, 1024, False, 1, 1)]:
+        layout = lt.get_blocksparse_layout(out_f, in_f, f"pixelfly(block_size=64, stretch={stretch})")
+        forward_indices, backward_indices = lt.get_indices_from_layout(layout)
+        assert shared_list_group(forward_indices, backward_indices.shape[1]) == out_group, (out_f, in_f, stretch)
+        assert shared_input_group(backward_indices) == in_group, (out_f, in_f, stretch)
+
+
 def test_shared_list_run_of_pixelfly_layouts():
     """runs of consecutive output blocks with one list of input blocks: stretched PixelFly on a tall matrix repeats every list
     out_blocks / in_blocks times, the tiled form and square matrices have none; the cached value follows in-place changes"""
