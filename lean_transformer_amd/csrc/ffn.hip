@@ -198,7 +198,10 @@ int linear_forward_impl(const lt_linear& lin, int64_t T, int dtype, const void* 
   p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
   p.sp.backward_indices = lin.backward_indices; p.sp.act = x; p.sp.ld_act = in; p.sp.weight = lin.weight;
   p.sp.out_group = group_length(lin.out_group); p.sp.out_stride = group_stride(lin.out_group);
-  p.sp.walk_run = walk_run_for(lin.in_features / lin.block, lin.out_features / lin.block, lin.blocks_per_out);
+  // (a tiled layout, known by its strided runs, lists the blocks of one tile of the square pattern together: as listed is
+  // the order in which the groups that share an activation block read it close together)
+  p.sp.walk_run = group_stride(lin.in_group) > 1
+                      ? 0 : walk_run_for(lin.in_features / lin.block, lin.out_features / lin.block, lin.blocks_per_out);
   bool two_passes = gated && !(dtype == LT_BF16 && lt_sparse_mfma_supported(p, kind));
   if (gated && !two_passes) {
     // Gate and linear output blocks have index lists of their own; the bf16 walk for 64 x 64 blocks pairs them inside one
@@ -285,7 +288,8 @@ int linear_backward_impl(const lt_linear& lin, int64_t T, int dtype, const void*
       p.sp.mode = SPARSE_DX; p.sp.block = lin.block; p.sp.blocks_per_out = lin.blocks_per_out;
       p.sp.blocks_per_in = lin.blocks_per_in; p.sp.forward_indices = lin.forward_indices;
       p.sp.backward_indices = lin.backward_indices; p.sp.act = dy; p.sp.ld_act = out; p.sp.weight = lin.weight;
-      p.sp.walk_run = walk_run_for(lin.out_features / lin.block, lin.in_features / lin.block, lin.blocks_per_in);
+      p.sp.walk_run = group_stride(lin.out_group) > 1
+                          ? 0 : walk_run_for(lin.out_features / lin.block, lin.in_features / lin.block, lin.blocks_per_in);
       if (kind_dx == EPI_ACT_BWD && act_colsum && (*act_colsum_rows = lt_gemm_colsum_rows(p, dtype, io_dtype)) > 0)
         p.epi.colsum = act_colsum;
       LT_TRY(lt_launch_gemm_sparse(p, kind_dx, dtype, io_dtype, stream));
