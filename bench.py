@@ -7,8 +7,8 @@ A step is one forward + backward of the module on a resident synthetic batch (pa
 K steps are timed by wall clock; the same K steps are then repeated with a HIP event pair around every kernel launch
 (recorded by the library on the launch stream) and `roofline` is computed from the GEMM launches of that pass;
 `cpu_baseline` times the CPU oracle (tests' checker, not the product) on a bounded sample of the same workload.
-The default run also measures configurations 2 and 4 (about a second of GPU time each) and reports them under
-`extra_configs` of the same line; `--config c4t` is configuration 4 with the reference's default layout (stretch=False);
+The default run also measures configurations 2, 4 and 4 with the reference's default layout (c4t: stretch=False), about a
+second of GPU time each, and reports them under `extra_configs` of the same line;
 `--config c5` times the full GPT train step of configuration 5 (the stock-PyTorch model of tests/gpt_harness.py around the
 FFN kernels).
 """
@@ -484,7 +484,7 @@ def main():
         del run, ffn, x, dy
         torch.cuda.empty_cache()
         extra = {}
-        for name in ("c2", "c4"):
+        for name in ("c2", "c4", "c4t"):
             other = run_ffn_config(torch, lt, nat, name, args.steps, args.warmup, device)
             entry = summarise(other, name)
             entry["config"] = {"workload": other["cfg"]["name"], "tokens": other["tokens"], "hidden": other["cfg"]["hidden"],
