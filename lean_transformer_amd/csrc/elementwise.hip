@@ -202,6 +202,54 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(int64_t T, int H, const TX*
   }
 }
 
+// Rows wider than the register-resident kernels take (hidden > 8192), any alignment: the same arithmetic with the columns in
+// a loop.  dx: a workgroup per row (grid-stride), two passes over the row; parameter gradients: one column per thread over a
+// slice of rows, one partial (dweight, dbias) row per slice.
+template <typename TX, typename TDY, typename TDX>
+__global__ __launch_bounds__(256) void ln_bwd_dx_wide_kernel(int64_t T, int H, const TX* __restrict__ x,
+                                                              const float* __restrict__ stats, const float* __restrict__ w,
+                                                              const TDY* __restrict__ dy,
+                                                              const TDX* __restrict__ residual_grad, TDX* __restrict__ dx) {
+  __shared__ float red[8];
+  const float inv_h = 1.0f / (float)H;
+  for (int64_t row = blockIdx.x; row < T; row += gridDim.x) {
+    const float mean = stats[row * 2], rstd = stats[row * 2 + 1];
+    const TX* xr = x + row * H;
+    const TDY* dyr = dy + row * H;
+    float s1 = 0.f, s2 = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) {
+      const float dxh = ldf(dyr, c) * w[c];
+      s1 += dxh;
+      s2 += dxh * ((ldf(xr, c) - mean) * rstd);
+    }
+    block_sum2(s1, s2, red);
+    const float c1 = s1 * inv_h, c2 = s2 * inv_h;
+    for (int c = threadIdx.x; c < H; c += 256) {
+      const float xh = (ldf(xr, c) - mean) * rstd;
+      float v = rstd * (ldf(dyr, c) * w[c] - c1 - xh * c2);
+      if (residual_grad) v += ldf(residual_grad, row * H + c);
+      stf(dx, row * H + c, v);
+    }
+  }
+}
+
+template <typename TX, typename TDY>
+__global__ __launch_bounds__(256) void ln_bwd_param_wide_kernel(int64_t T, int H, const TX* __restrict__ x,
+                                                                 const float* __restrict__ stats, const TDY* __restrict__ dy,
+                                                                 int64_t rows_per_slice, float* __restrict__ partial) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= H) return;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice, r1 = min(T, r0 + rows_per_slice);
+  float pw = 0.f, pb = 0.f;
+  for (int64_t r = r0; r < r1; r++) {
+    const float g = ldf(dy, r * H + c);
+    pw += g * ((ldf(x, r * H + c) - stats[r * 2]) * stats[r * 2 + 1]);
+    pb += g;
+  }
+  partial[((int64_t)blockIdx.y * 2) * H + c] = pw;
+  partial[((int64_t)blockIdx.y * 2 + 1) * H + c] = pb;
+}
+
 // Vectorised LayerNorm backward (hidden % 4 == 0, hidden <= 8192, 16-byte aligned rows), split in two so that neither half
 // has to keep per-column partial sums next to a cached row:
 //   ln_bwd_dx_kernel      one wavefront per row; dy and x of the row live in registers, the two row sums go through
@@ -675,7 +723,6 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
                    const void* dy, int dx_dtype, const void* residual_grad, void* dx, float* dweight, float* dbias,
                    void* workspace, size_t workspace_bytes, hipStream_t stream, ColReduceQueue* defer) {
   LT_REQUIRE(T > 0 && H > 0 && x && stats && w && dy, LT_ERR_BAD_ARG, "layernorm backward: bad arguments");
-  LT_REQUIRE(H <= 256 * LNB_MAXC, LT_ERR_UNSUPPORTED, "layernorm backward: hidden size %d above %d", H, 256 * LNB_MAXC);
   LT_REQUIRE((dweight == nullptr) == (dbias == nullptr), LT_ERR_BAD_ARG, "layernorm backward: pass both dweight and dbias or neither");
   float* partial = dweight ? (float*)workspace : nullptr;
   LtProfileScope scope("layernorm_bwd", 0.0,
@@ -686,8 +733,9 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
   const bool vec = (H & 3) == 0 && H <= 64 * 4 * LN_MAXV && lt_aligned(x, 16) && lt_aligned(dy, 16) && lt_aligned(w, 16) &&
                    (!dx || lt_aligned(dx, 16)) && (!residual_grad || lt_aligned(residual_grad, 16)) &&
                    (!partial || lt_aligned(partial, 16));
-  // partial (dweight, dbias) rows of the path taken: one pair per row slice (vectorised) or per workgroup (any-shape)
-  int partial_rows = vec ? ln_bwd_slices(T) : ln_bwd_blocks(T);
+  const bool wide = H > 256 * LNB_MAXC;  // wider than the register-resident kernels take
+  // partial (dweight, dbias) rows of the path taken: one pair per row slice (vectorised, wide) or per workgroup (any-shape)
+  int partial_rows = (vec || wide) ? ln_bwd_slices(T) : ln_bwd_blocks(T);
   if (dweight) {
     const size_t need = (size_t)partial_rows * 2 * (size_t)H * sizeof(float);
     LT_REQUIRE(workspace && workspace_bytes >= need, LT_ERR_WORKSPACE,
@@ -733,6 +781,40 @@ int lt_ln_backward(int64_t T, int H, int x_dtype, const void* x, const float* st
         default: LT_LNB_PARAM(bf16, bf16); break;
       }
 #undef LT_LNB_PARAM
+      LT_LAUNCH_CHECK();
+    }
+  } else if (wide) {
+    if (dx) {
+      dim3 grid((unsigned)ln_bwd_blocks(T)), block(256);
+#define LT_LNB_WIDE(TX, TDY, TDX)                                                                                          \
+  hipLaunchKernelGGL((ln_bwd_dx_wide_kernel<TX, TDY, TDX>), grid, block, 0, stream, T, H, (const TX*)x, stats, w, (const TDY*)dy, \
+                     (const TDX*)residual_grad, (TDX*)dx)
+      switch (key) {
+        case 0: LT_LNB_WIDE(float, float, float); break;
+        case 1: LT_LNB_WIDE(float, float, bf16); break;
+        case 2: LT_LNB_WIDE(float, bf16, float); break;
+        case 3: LT_LNB_WIDE(float, bf16, bf16); break;
+        case 4: LT_LNB_WIDE(bf16, float, float); break;
+        case 5: LT_LNB_WIDE(bf16, float, bf16); break;
+        case 6: LT_LNB_WIDE(bf16, bf16, float); break;
+        default: LT_LNB_WIDE(bf16, bf16, bf16); break;
+      }
+#undef LT_LNB_WIDE
+      LT_LAUNCH_CHECK();
+    }
+    if (partial) {
+      const int64_t rps = (T + partial_rows - 1) / partial_rows;
+      dim3 grid(blocks_for(H, 256), partial_rows), block(256);
+#define LT_LNB_WIDE_PARAM(TX, TDY)                                                                                         \
+  hipLaunchKernelGGL((ln_bwd_param_wide_kernel<TX, TDY>), grid, block, 0, stream, T, H, (const TX*)x, stats, (const TDY*)dy, \
+                     rps, partial)
+      switch (key >> 1) {
+        case 0: LT_LNB_WIDE_PARAM(float, float); break;
+        case 1: LT_LNB_WIDE_PARAM(float, bf16); break;
+        case 2: LT_LNB_WIDE_PARAM(bf16, float); break;
+        default: LT_LNB_WIDE_PARAM(bf16, bf16); break;
+      }
+#undef LT_LNB_WIDE_PARAM
       LT_LAUNCH_CHECK();
     }
   } else {

@@ -357,8 +357,6 @@ int check_ffn_desc(const lt_ffn_desc* d) {
              (long long)d->tokens, d->hidden, d->intermediate);
   LT_TRY(check_dtype(d->io_dtype, "ffn io_dtype"));
   LT_TRY(check_dtype(d->compute_dtype, "ffn compute_dtype"));
-  // the LayerNorm kernels hold a row in registers (backward has no strided variant): refuse wider rows before any work
-  LT_REQUIRE(d->hidden <= 8192, LT_ERR_UNSUPPORTED, "ffn: hidden size %d exceeds 8192, the widest row the LayerNorm kernels take", d->hidden);
   LT_REQUIRE(d->act >= 0 && d->act < LT_ACT_COUNT, LT_ERR_UNSUPPORTED, "ffn: unknown activation %d", d->act);
   LT_REQUIRE(d->ln_weight && d->ln_bias, LT_ERR_BAD_ARG, "ffn: LayerNorm parameters missing");
   LT_REQUIRE((d->post_ln_weight == nullptr) == (d->post_ln_bias == nullptr), LT_ERR_BAD_ARG, "ffn: post-LN needs weight and bias");

@@ -418,6 +418,30 @@ def test_ffn_empty_batch(dtype):
         assert g.shape == prm.shape and g.dtype == prm.dtype and not g.any()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ffn_with_rows_wider_than_the_register_resident_layernorm(dtype):
+    """hidden 12288 (rows of more than 8192 elements: the LayerNorm kernels walk the columns in a loop)"""
+    torch.manual_seed(11)
+    hidden, inter, tokens = 12288, 512, 96
+    ffn = lt.LeanFFN(hidden, inter, gated=True, layer_norm_eps=1e-5)
+    with torch.no_grad():
+        ffn.pre_layer_norm.weight.uniform_(0.5, 1.5)
+        ffn.pre_layer_norm.bias.normal_(std=0.2)
+        ffn.i2h_proj.bias.normal_(std=0.1)
+        ffn.h2o_proj.bias.normal_(std=0.1)
+    x, dy = torch.randn(tokens, hidden), torch.randn(tokens, hidden)
+    p = oracle_params(ffn)
+    y_ref, dx_ref, g_ref = run_oracle(p, x, dy)
+    ffn = ffn.to(DEV).to(dtype)
+    xd = x.to(DEV).to(dtype).requires_grad_(True)
+    y = ffn(xd)
+    grads = torch.autograd.grad(y, [xd, *module_tensors(ffn)], dy.to(DEV).to(dtype))
+    assert_close(y, y_ref, dtype, "y")
+    assert_close(grads[0], dx_ref, dtype, "dx")
+    for i, (a, b) in enumerate(zip(grads[1:], g_ref)):
+        assert_close(a, b, dtype, f"param grad {i}")
+
+
 def test_ffn_refuses_what_it_cannot_run():
     """loud failures, no fallback: half precision, an activation the kernels do not have, a plug-in matmul op"""
     ffn = lt.LeanFFN(256, 512).to(DEV)

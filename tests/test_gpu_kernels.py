@@ -157,7 +157,7 @@ def test_layernorm_forward(tokens, hidden, x_dtype, y_dtype):
     assert torch.allclose(stats[:, 1].cpu(), torch.rsqrt(x.float().var(-1, unbiased=False) + 1e-5), rtol=1e-4)
 
 
-@pytest.mark.parametrize("tokens,hidden", [(37, 32), (300, 768), (2100, 256), (3, 10), (4, 8192)])
+@pytest.mark.parametrize("tokens,hidden", [(37, 32), (300, 768), (2100, 256), (3, 10), (4, 8192), (3, 12288), (70, 8200), (5, 8202)])
 @pytest.mark.parametrize("x_dtype,dy_dtype,dx_dtype", [(torch.float32, torch.float32, torch.float32),
                                                        (torch.bfloat16, torch.bfloat16, torch.bfloat16),
                                                        (torch.float32, torch.bfloat16, torch.float32)])
