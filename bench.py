@@ -40,6 +40,10 @@ CONFIGS = {
     "c4": dict(batch=2, seq=2048, hidden=4096, inter=16384, gated=True, std=0.02, dropout=0.0, dtype="bf16", sparse=True,
                name="config4: LeanFFN PixelFly (64x64 blocks, stretch, density 7/64) + rank-128 low-rank GeGLU fwd+bwd, "
                     "hidden 4096, intermediate 16384, x [2,2048,4096], bf16"),
+    # config 3 on the float16 twin of the library (same kernels, IEEE binary16 operands on the f16 matrix instruction)
+    "c3h": dict(batch=2, seq=2048, hidden=4096, inter=16384, gated=True, std=0.01, dropout=0.0, dtype="fp16", sparse=False,
+                name="config3 in float16: LeanFFN dense GeGLU fwd+bwd, hidden 4096, intermediate 16384, x [2,2048,4096] fp32 "
+                     "residual stream, fp16 weights/activations, fp32 accumulation, dropout 0"),
     # config 4 with the reference's default layout (pixelfly tiles the square butterfly instead of stretching it: no runs of
     # blocks with one list, every product is a walk over the index tables)
     "c4t": dict(batch=2, seq=2048, hidden=4096, inter=16384, gated=True, std=0.02, dropout=0.0, dtype="bf16", sparse=True,
@@ -73,8 +77,8 @@ def build_workload(torch, lt, cfg, device):
             ffn.h2o_proj.bias.zero_()
     dy = torch.randn(cfg["batch"], cfg["seq"], hidden, generator=g)
     ffn = ffn.to(device)
-    if cfg["dtype"] == "bf16":
-        ffn = ffn.to(torch.bfloat16)
+    if cfg["dtype"] != "fp32":
+        ffn = ffn.to(torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float16)
     return ffn, x.to(device).requires_grad_(True), dy.to(device)
 
 
@@ -169,7 +173,9 @@ def measured_traffic(config):
     configuration (written when that summary is refreshed), with the algorithmic bytes of the same launches and where the
     figure comes from: the summary records the hash of the kernel sources it was measured on, and `stale` says whether the
     tree's kernels still are those.  (None, None, None) when the configuration has no such summary."""
-    counted = config != "c4t"  # the default-layout variant of config 4 has config 4's algorithmic bytes and no counter run
+    # the default-layout variant of config 4 and the float16 variant of config 3 have their base configuration's
+    # algorithmic bytes and no counter run of their own
+    counted = config not in ("c4t", "c3h")
     path = os.path.join(ROOT, "profiles", f"leanffn_config{config[1:2]}_gemm_hbm_traffic.json")
     if not os.path.exists(path):
         return None, None, None
@@ -276,7 +282,7 @@ def run_ffn_config(torch, lt, nat, name, steps, warmup, device):
     peak_mb = (torch.cuda.max_memory_allocated() - base) / 2**20
     del y
 
-    lib = nat.lib()
+    lib = nat.lib(torch.float16 if cfg["dtype"] == "fp16" else None)
     lib.lt_profile_enable(0)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -296,7 +302,7 @@ def run_ffn_config(torch, lt, nat, name, steps, warmup, device):
     torch.cuda.synchronize()
     elapsed_events = time.perf_counter() - t0
     lib.lt_profile_enable(0)
-    kernels = nat.profile_read()
+    kernels = nat.profile_read(lib)
     lib.lt_profile_reset()
     return dict(cfg=cfg, name=name, tokens=tokens, ffn=ffn, x=x, dy=dy, ms_per_step=elapsed / steps * 1e3,
                 ms_events=elapsed_events / steps * 1e3, kernels=kernels, saved_mb=saved_mb, peak_mb=peak_mb)
@@ -305,7 +311,7 @@ def run_ffn_config(torch, lt, nat, name, steps, warmup, device):
 def summarise(run, config_name):
     """throughput, kernel table and roofline object of one run_ffn_config result"""
     cfg, kernels, tokens, ms_per_step = run["cfg"], run["kernels"], run["tokens"], run["ms_per_step"]
-    peak = PEAK_BF16_TFLOPS if cfg["dtype"] == "bf16" else PEAK_FP32_TFLOPS
+    peak = PEAK_FP32_TFLOPS if cfg["dtype"] == "fp32" else PEAK_BF16_TFLOPS  # bf16 and fp16 share one dense peak
     tflops = algorithmic_flops(cfg) / (ms_per_step * 1e-3) / 1e12
     gemm = [k for k in kernels if k[0].startswith(("gemm_", "blocksparse_"))]
     gemm_flops, gemm_ms, gemm_launches = sum(k[3] for k in gemm), sum(k[2] for k in gemm), sum(k[1] for k in gemm)
@@ -451,7 +457,7 @@ def main():
         "metric": METRIC, "value": summary["value"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": summary["ms_per_step"],
         "ms_per_step_with_kernel_events": summary["ms_per_step_with_kernel_events"], "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if cfg["dtype"] == "bf16" else "f32", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": {"bf16": "bf16", "fp16": "f16", "fp32": "f32"}[cfg["dtype"]], "data": "synthetic",
         "config": {"workload": cfg["name"], "tokens": tokens, "hidden": hidden, "intermediate": inter},
         "tflops": summary["tflops"], "mfma_util_pct": summary["mfma_util_pct"],
         "peak_activation_mb": summary["peak_activation_mb"], "saved_activation_mb": summary["saved_activation_mb"],

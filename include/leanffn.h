@@ -37,7 +37,12 @@ typedef enum lt_status {
   LT_ERR_HIP = 4          /* a HIP runtime call or kernel launch failed */
 } lt_status;
 
-typedef enum lt_dtype { LT_F32 = 0, LT_BF16 = 1 } lt_dtype;
+/* Element types.  The 16-bit type is fixed when the library is compiled: libleanffn.so computes in bfloat16 and accepts
+ * LT_F32 and LT_BF16; libleanffn_f16.so is the same sources compiled with -DLT_HALF_IS_FP16 (IEEE binary16 operands on
+ * v_mfma_f32_32x32x16_f16, the same kernels otherwise) and accepts LT_F32 and LT_F16.  Either library refuses the other's
+ * 16-bit code with LT_ERR_BAD_ARG; a process may load both (they share no state).  Accumulation is fp32 in both; fp16's
+ * range is the caller's to manage (loss scaling), as under torch.autocast(float16) in the reference. */
+typedef enum lt_dtype { LT_F32 = 0, LT_BF16 = 1, LT_F16 = 2 } lt_dtype;
 
 /* Activations evaluated in registers, value and derivative: the reference's gelu_fused (tanh form, lean_transformer/utils.py:24-38)
  * and the closed-form entries of transformers.activations.ACT2FN, the table the reference's ACT2FN extends (utils.py:80).

@@ -1,6 +1,10 @@
-"""Builds lean_transformer_amd/csrc/libleanffn.so from the HIP sources with hipcc for gfx950 (cross-compiles without a GPU).
+"""Builds lean_transformer_amd/csrc/libleanffn.so and libleanffn_f16.so from the HIP sources with hipcc for gfx950
+(cross-compiles without a GPU).  The two libraries are the same sources with the 16-bit element type fixed at compile time:
+bfloat16 in the first, IEEE binary16 (-DLT_HALF_IS_FP16) in the second.
 
-    python -m lean_transformer_amd._build
+    python -m lean_transformer_amd._build            # both
+    python -m lean_transformer_amd._build --bf16     # libleanffn.so only
+    python -m lean_transformer_amd._build --f16      # libleanffn_f16.so only
 """
 import os
 import subprocess
@@ -34,20 +38,34 @@ def _run(cmd):
     return proc.stdout
 
 
+F16_LIB_PATH = os.path.join(CSRC, "libleanffn_f16.so")
 TILE_TIMING_LIB_PATH = os.path.join(CSRC, "libleanffn_tile_timing.so")
 
 
-def build(verbose: bool = False, extra_flags=(), tile_timing: bool = False) -> str:
+def build_all(verbose: bool = False) -> list:
+    """Both libraries, their translation units compiled side by side; returns their paths."""
+    with ThreadPoolExecutor(max_workers=2) as pool:
+        futures = [pool.submit(build, verbose=verbose, f16=f16, workers=4) for f16 in (False, True)]
+        return [f.result() for f in futures]
+
+
+def build(verbose: bool = False, extra_flags=(), tile_timing: bool = False, f16: bool = False, workers: int = 8) -> str:
     """Compile every translation unit (in parallel) and link the shared library; returns its path.
+
+    f16: build libleanffn_f16.so, whose 16-bit element type is IEEE binary16, instead of the bfloat16 library.
 
     tile_timing: build the instrumented library instead (csrc/libleanffn_tile_timing.so, -DLT_TILE_TIMING: the copy-based
     GEMM kernels record per-workgroup phase timestamps; read by tile_timing.py at the repository root).  Never loaded by the
     package itself."""
     hipcc = _hipcc()
-    suffix = ".tile_timing.o" if tile_timing else ".o"
-    lib_path = TILE_TIMING_LIB_PATH if tile_timing else LIB_PATH
+    if tile_timing and f16:
+        raise ValueError("the instrumented library is built for bfloat16 only")
+    suffix = ".tile_timing.o" if tile_timing else ".f16.o" if f16 else ".o"
+    lib_path = TILE_TIMING_LIB_PATH if tile_timing else F16_LIB_PATH if f16 else LIB_PATH
     if tile_timing:
         extra_flags = (*extra_flags, "-DLT_TILE_TIMING")
+    if f16:
+        extra_flags = (*extra_flags, "-DLT_HALF_IS_FP16")
     objects = [os.path.join(CSRC, src.replace(".hip", suffix)) for src in SOURCES]
 
     def compile_one(pair):
@@ -56,11 +74,16 @@ def build(verbose: bool = False, extra_flags=(), tile_timing: bool = False) -> s
         if verbose and out.strip():
             print(out)
 
-    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, 8, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, workers, len(SOURCES))) as pool:
         list(pool.map(compile_one, zip(SOURCES, objects)))
     _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objects, "-o", lib_path])
     return lib_path
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv, tile_timing="--tile-timing" in sys.argv))
+    if "--tile-timing" in sys.argv:
+        print(build(verbose="-v" in sys.argv, tile_timing=True))
+    elif "--bf16" in sys.argv or "--f16" in sys.argv:
+        print(build(verbose="-v" in sys.argv, f16="--f16" in sys.argv))
+    else:
+        print(*build_all(verbose="-v" in sys.argv), sep="\n")

@@ -1,8 +1,9 @@
-"""ctypes binding of csrc/libleanffn.so (declarations: include/leanffn.h).
+"""ctypes binding of csrc/libleanffn.so and csrc/libleanffn_f16.so (declarations: include/leanffn.h).
 
-The library is the only compute backend of this package: there is no fallback.  ``lib()`` raises if the shared object has
-not been built (``python -m lean_transformer_amd._build``), and every call raises ``RuntimeError`` with the library's own
-message when it returns a non-zero status.
+The two libraries are the same kernels with the 16-bit element type fixed at compile time (bfloat16 / IEEE binary16);
+``lib(dtype)`` picks the one that computes in ``dtype``.  They are the only compute backend of this package: there is no
+fallback.  ``lib()`` raises if the shared object has not been built (``python -m lean_transformer_amd._build``), and every
+call raises ``RuntimeError`` with the library's own message when it returns a non-zero status.
 """
 import ctypes
 import os
@@ -12,9 +13,10 @@ from typing import Optional
 import torch
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libleanffn.so")
+F16_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libleanffn_f16.so")
 
-LT_F32, LT_BF16 = 0, 1
-_DTYPES = {torch.float32: LT_F32, torch.bfloat16: LT_BF16}
+LT_F32, LT_BF16, LT_F16 = 0, 1, 2
+_DTYPES = {torch.float32: LT_F32, torch.bfloat16: LT_BF16, torch.float16: LT_F16}
 
 # every function include/leanffn.h declares; the not-gpu tests check that the built library exports all of them
 EXPORTED_SYMBOLS = (
@@ -67,7 +69,7 @@ class LtFfnGrads(ctypes.Structure):
                 ("post_ln_bias", c_void_p), ("i2h", LtLinearGrads), ("h2o", LtLinearGrads)]
 
 
-_lib = None
+_libs = {}
 
 
 def _declare(lib):
@@ -118,26 +120,33 @@ def _declare(lib):
 def available() -> bool:
     """whether the built library is there (the only caller: the stock-op path's choice of dropout mask; every kernel path
     calls lib() and fails loudly without it)"""
-    return _lib is not None or os.path.exists(LIB_PATH)
+    return bool(_libs) or os.path.exists(LIB_PATH)
 
 
-def lib():
-    """The loaded library; raises if it was never built."""
-    global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
+def lib(*dtypes: Optional[torch.dtype]):
+    """The loaded library that computes in the given dtypes: libleanffn_f16.so when one of them is float16, libleanffn.so
+    otherwise (float32 work runs on the same kernels in either).  Raises if the library was never built, and when float16
+    and bfloat16 meet in one call (no kernel mixes them)."""
+    f16 = torch.float16 in dtypes
+    if f16 and torch.bfloat16 in dtypes:
+        raise TypeError("float16 and bfloat16 tensors in one call: the kernels compute in one 16-bit type at a time")
+    path = F16_LIB_PATH if f16 else LIB_PATH
+    loaded = _libs.get(path)
+    if loaded is None:
+        if not os.path.exists(path):
             raise RuntimeError(
-                f"{LIB_PATH} is missing: the HIP kernels of lean_transformer_amd are not built. "
+                f"{path} is missing: the HIP kernels of lean_transformer_amd are not built. "
                 "Run `python -m lean_transformer_amd._build` (needs hipcc; cross-compiles for gfx950 without a GPU).")
-        loaded = ctypes.CDLL(LIB_PATH)
+        loaded = ctypes.CDLL(path)
         _declare(loaded)
-        _lib = loaded
-    return _lib
+        _libs[path] = loaded
+    return loaded
 
 
-def check(status: int, what: str):
+def check(status: int, what: str, library=None):
+    """raise with the message of the library that returned ``status`` (the bfloat16 one unless ``library`` is given)"""
     if status != 0:
-        message = lib().lt_last_error().decode("utf-8", "replace")
+        message = (library or lib()).lt_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"{what} failed (lt_status {status}): {message}")
 
 
@@ -145,7 +154,7 @@ def dtype_code(dtype: torch.dtype) -> int:
     try:
         return _DTYPES[dtype]
     except KeyError:
-        raise TypeError(f"the HIP kernels take float32 and bfloat16 tensors, not {dtype}") from None
+        raise TypeError(f"the HIP kernels take float32, bfloat16 and float16 tensors, not {dtype}") from None
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -179,10 +188,12 @@ def workspace(nbytes: int, device: torch.device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
-def profile_read():
-    """[(kernel tag, launches, total ms, algorithmic flops, algorithmic bytes)] recorded since the last lt_profile_reset"""
+def profile_read(library=None):
+    """[(kernel tag, launches, total ms, algorithmic flops, algorithmic bytes)] recorded by ``library`` (the bfloat16 one
+    unless given) since the last lt_profile_reset"""
+    library = library or lib()
     entries = (LtProfileEntry * 64)()
-    n = lib().lt_profile_read(entries, 64)
+    n = library.lt_profile_read(entries, 64)
     if n < 0:
-        check(-n, "lt_profile_read")
+        check(-n, "lt_profile_read", library)
     return [(e.name.decode(), e.launches, e.ms, e.flops, e.bytes) for e in entries[:min(n, 64)]]

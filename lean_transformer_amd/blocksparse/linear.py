@@ -124,8 +124,8 @@ def compute_dtype_for(weight: torch.Tensor) -> torch.dtype:
     """dtype of GEMM operands: the autocast dtype when autocast is on (as F.linear would use), else the weight's dtype"""
     if torch.is_autocast_enabled("cuda"):
         dtype = torch.get_autocast_dtype("cuda")
-        if dtype != torch.bfloat16:
-            raise NotImplementedError(f"autocast to {dtype}: the HIP kernels compute in bfloat16 or float32")
+        if dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"autocast to {dtype}: the HIP kernels compute in bfloat16, float16 or float32")
         return dtype
     return weight.dtype
 
@@ -280,8 +280,9 @@ class _GeneralizedLinear(torch.autograd.Function):
         y = torch.empty(tokens, desc.out_features, dtype=dtype, device=device)
         hid = torch.empty(tokens, desc.lowrank, dtype=dtype, device=device) if desc.lowrank else None
         if tokens > 0:
-            nat.check(nat.lib().lt_linear_forward(desc, tokens, nat.dtype_code(dtype), nat.ptr(x), nat.ptr(y), nat.ptr(hid),
-                                                  nat.current_stream(device)), "lt_linear_forward")
+            lib = nat.lib(dtype)
+            nat.check(lib.lt_linear_forward(desc, tokens, nat.dtype_code(dtype), nat.ptr(x), nat.ptr(y), nat.ptr(hid),
+                                            nat.current_stream(device)), "lt_linear_forward", lib)
         ctx.save_for_backward(input, hid, main_weight, lowrank_first, lowrank_second, forward_indices, backward_indices)
         ctx._dtype, ctx._has_bias = dtype, bias is not None
         return y.view(*input.shape[:-1], desc.out_features)
@@ -309,11 +310,11 @@ class _GeneralizedLinear(torch.autograd.Function):
         grads.weight, grads.bias, grads.lowrank_first, grads.lowrank_second = (nat.ptr(dw), nat.ptr(db), nat.ptr(dl1),
                                                                                nat.ptr(dl2))
         if tokens > 0:
-            lib = nat.lib()
+            lib = nat.lib(dtype)
             ws = nat.workspace(lib.lt_linear_backward_workspace_bytes(desc, tokens, nat.dtype_code(dtype)), device)
             nat.check(lib.lt_linear_backward(desc, tokens, nat.dtype_code(dtype), nat.ptr(x), nat.ptr(dy), nat.ptr(hid),
                                              nat.ptr(dx), grads, nat.ptr(ws), ws.numel(), nat.current_stream(device)),
-                      "lt_linear_backward")
+                      "lt_linear_backward", lib)
         else:
             for g in (dw, db, dl1, dl2):
                 if g is not None:

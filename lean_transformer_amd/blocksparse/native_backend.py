@@ -42,8 +42,9 @@ def blocksparse_matmul(input: torch.Tensor, weight: torch.Tensor, forward_indice
     y = torch.empty(x.shape[0], out_features, dtype=x.dtype, device=device)
     if x.shape[0] > 0:
         desc = _sparse_desc(w, fwd, None, out_features)
-        nat.check(nat.lib().lt_blocksparse_forward(desc, x.shape[0], nat.dtype_code(x.dtype), nat.ptr(x), nat.ptr(y),
-                                                    nat.current_stream(device)), "lt_blocksparse_forward")
+        lib = nat.lib(x.dtype)
+        nat.check(lib.lt_blocksparse_forward(desc, x.shape[0], nat.dtype_code(x.dtype), nat.ptr(x), nat.ptr(y),
+                                             nat.current_stream(device)), "lt_blocksparse_forward", lib)
     return y.view(*input.shape[:-1], out_features)
 
 
@@ -66,9 +67,10 @@ def blocksparse_matmul_backward(grad_output: torch.Tensor, input: torch.Tensor, 
     grad_weight = torch.empty_like(w) if weight_requires_grad else None
     if x.shape[0] > 0:
         desc = _sparse_desc(w, None, bwd, dy.shape[1])
-        nat.check(nat.lib().lt_blocksparse_backward(desc, x.shape[0], nat.dtype_code(x.dtype), nat.ptr(x), nat.ptr(dy),
-                                                     nat.ptr(grad_input), nat.ptr(grad_weight),
-                                                     nat.current_stream(device)), "lt_blocksparse_backward")
+        lib = nat.lib(x.dtype)
+        nat.check(lib.lt_blocksparse_backward(desc, x.shape[0], nat.dtype_code(x.dtype), nat.ptr(x), nat.ptr(dy),
+                                              nat.ptr(grad_input), nat.ptr(grad_weight), nat.current_stream(device)),
+                  "lt_blocksparse_backward", lib)
     else:
         if grad_weight is not None:
             grad_weight.zero_()

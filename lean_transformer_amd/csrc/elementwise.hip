@@ -890,7 +890,9 @@ extern "C" int lt_layernorm_backward_static(int64_t tokens, int32_t hidden, int3
                                             void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   for (int d : {x_dtype, dy_dtype, dx_dtype})
-    LT_REQUIRE(d == LT_F32 || d == LT_BF16, LT_ERR_BAD_ARG, "layernorm backward (static scratch): unknown dtype %d", d);
+    LT_REQUIRE(d == LT_F32 || d == LT_BF16, LT_ERR_BAD_ARG,
+               "layernorm backward (static scratch): dtype code %d is not one of this library's (fp32 = %d, " LT_HALF_NAME " = %d)", d,
+               (int)LT_F32, (int)LT_BF16);
   void* ptr = nullptr;
   if (dweight) LT_TRY(static_scratch_for(stream, &ptr));
   const int status = lt_ln_backward(tokens, hidden, x_dtype, x, stats, weight, dy_dtype, dy, dx_dtype, residual_grad, dx,

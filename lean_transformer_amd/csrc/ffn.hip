@@ -25,7 +25,7 @@ void lt_set_error(const char* fmt, ...) {
 }
 
 extern "C" const char* lt_last_error(void) { return g_error; }
-extern "C" const char* lt_version(void) { return "libleanffn 0.1.0 (gfx950)"; }
+extern "C" const char* lt_version(void) { return "libleanffn 0.1.0 (gfx950, 16-bit type " LT_HALF_NAME ")"; }
 
 namespace {
 
@@ -43,7 +43,8 @@ struct Bump {
 };
 
 int check_dtype(int d, const char* what) {
-  LT_REQUIRE(d == LT_F32 || d == LT_BF16, LT_ERR_BAD_ARG, "%s: unknown dtype %d", what, d);
+  LT_REQUIRE(d == LT_F32 || d == LT_BF16, LT_ERR_BAD_ARG, "%s: dtype code %d is not one of this library's (fp32 = %d, " LT_HALF_NAME " = %d)", what,
+             d, (int)LT_F32, (int)LT_BF16);
   return LT_OK;
 }
 

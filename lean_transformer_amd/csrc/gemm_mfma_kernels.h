@@ -349,7 +349,7 @@ void gemm_bf16_kernel(GemmProblem p, int tiles_m, int tiles_n) {
       for (int i = 0; i < FM; i++)
 #pragma unroll
         for (int j = 0; j < FN_IN; j++)
-          acc[i][j0 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j0 + j], 0, 0, 0);
+          acc[i][j0 + j] = LT_MFMA_32X32X16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j0 + j]);
       if (kk + 1 < BK / 16) SchedInterleave<FRAG_READS, FM * FN_IN>::run();
     }
   };
@@ -1363,7 +1363,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(GemmProblem problem,
 #pragma unroll
     for (int q = 0; q < 16; q++) {
       const int x = ORDER[q][0], y = ORDER[q][1];
-      acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y], 0, 0, 0);
+      acc[x][y] = LT_MFMA_32X32X16(a[x], b[y], acc[x][y]);
     }
   };
   constexpr int FRAG_READS = FM * (A_KM ? 1 : 2) + FN * (B_KM ? 1 : 2);

@@ -7,8 +7,21 @@
 
 #include "../../include/leanffn.h"
 
+// The 16-bit element type of this build.  The sources name it bf16 throughout; compiled with -DLT_HALF_IS_FP16 the same
+// name stands for IEEE binary16, the dtype code the library accepts for it is LT_F16 instead of LT_BF16, and the matrix
+// instruction is the f16 one of the same shape.  Nothing else depends on the format: conversions are casts, the LDS and
+// copy paths move 16-bit words, every accumulator is fp32.
+#ifdef LT_HALF_IS_FP16
+typedef _Float16 bf16;
+#define LT_BF16 LT_F16
+#define LT_HALF_NAME "fp16"
+#define LT_MFMA_32X32X16(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0)
+#else
 typedef __bf16 bf16;
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+#define LT_HALF_NAME "bf16"
+#define LT_MFMA_32X32X16(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
+#endif
+typedef __attribute__((__vector_size__(8 * sizeof(bf16)))) bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;

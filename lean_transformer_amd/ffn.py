@@ -189,9 +189,9 @@ class _LeanFFN(torch.autograd.Function):
         act = ACT_KINDS[activation_kind(activation)]
         cdt = compute_dtype_for(i2h_weight)
         io = input.dtype
-        if io not in (torch.float32, torch.bfloat16) or (io == torch.bfloat16 and cdt != torch.bfloat16):
-            raise TypeError(f"LeanFFN: input dtype {io} with compute dtype {cdt} is not supported "
-                            "(float32 input with float32/bfloat16 weights, or bfloat16 input with bfloat16 weights)")
+        if io not in (torch.float32, torch.bfloat16, torch.float16) or (io != torch.float32 and cdt != io):
+            raise TypeError(f"LeanFFN: input dtype {io} with compute dtype {cdt} is not supported (float32 input with "
+                            "float32/bfloat16/float16 weights, or bfloat16/float16 input with weights of the same dtype)")
         hidden = input.shape[-1]
         x = input.detach().reshape(-1, hidden).contiguous()
         tokens = x.shape[0]
@@ -219,10 +219,10 @@ class _LeanFFN(torch.autograd.Function):
         if tokens > 0:
             saved = nat.LtFfnSaved(nat.ptr(pre_activation), nat.ptr(ln_stats), nat.ptr(post_ln_input), nat.ptr(i2h_hid),
                                    nat.ptr(h2o_hid))
-            lib = nat.lib()
+            lib = nat.lib(cdt)
             ws = nat.workspace(lib.lt_ffn_forward_workspace_bytes(desc), device)
             nat.check(lib.lt_ffn_forward(desc, nat.ptr(x), nat.ptr(y), saved, nat.ptr(ws), ws.numel(),
-                                         nat.current_stream(device)), "lt_ffn_forward")
+                                         nat.current_stream(device)), "lt_ffn_forward", lib)
             del ws, keep
         ctx.save_for_backward(
             input, pre_activation, ln_stats, post_ln_input, i2h_hid, h2o_hid, ln_weight, ln_bias,
@@ -316,10 +316,10 @@ class _LeanFFN(torch.autograd.Function):
             grads.h2o = nat.LtLinearGrads(nat.ptr(d_h2o_w), nat.ptr(d_h2o_b), nat.ptr(d_h2o_l1), nat.ptr(d_h2o_l2))
             saved = nat.LtFfnSaved(nat.ptr(pre_activation), nat.ptr(ln_stats), nat.ptr(post_ln_input), nat.ptr(i2h_hid),
                                    nat.ptr(h2o_hid))
-            lib = nat.lib()
+            lib = nat.lib(cdt)
             ws = nat.workspace(lib.lt_ffn_backward_workspace_bytes(desc), device)
             nat.check(lib.lt_ffn_backward(desc, nat.ptr(x), nat.ptr(dy), saved, grads, nat.ptr(ws), ws.numel(),
-                                          nat.current_stream(device)), "lt_ffn_backward")
+                                          nat.current_stream(device)), "lt_ffn_backward", lib)
             del ws, keep
         else:
             for g in outputs[1:]:

@@ -38,6 +38,8 @@ def cosine(got: torch.Tensor, ref: torch.Tensor) -> float:
 FP32_TOL = 1e-4   # max relative error, fp32 path
 BF16_TOL = 2e-2   # max relative error, bf16 path
 BF16_COS = 0.9999  # minimum cosine similarity, bf16 path
+FP16_TOL = 4e-3   # max relative error, fp16 path (11 significant bits against bf16's 8: the bf16 bar / 5)
+FP16_COS = 0.999996  # minimum cosine similarity, fp16 path (1 - cosine goes with the square of the error: 1e-4 / 25)
 
 
 def assert_close(got, ref, dtype, name=""):
@@ -54,7 +56,8 @@ def assert_close(got, ref, dtype, name=""):
         assert worst <= 0.0, f"{name}: an element is {worst:.3e} beyond 1e-4 * |ref| + 1e-5 * max|ref|"
     else:
         cos = cosine(got, ref)
-        assert err <= BF16_TOL and cos >= BF16_COS, f"{name}: max relative error {err:.3e}, cosine {cos:.6f}"
+        tol, floor = (FP16_TOL, FP16_COS) if dtype == torch.float16 else (BF16_TOL, BF16_COS)
+        assert err <= tol and cos >= floor, f"{name}: max relative error {err:.3e} (bar {tol}), cosine {cos:.7f} (bar {floor})"
 
 
 def assert_within_bf16_noise(named_got, named_truth, stock_runs, label="", depth=1):

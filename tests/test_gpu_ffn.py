@@ -443,10 +443,13 @@ def test_ffn_with_rows_wider_than_the_register_resident_layernorm(dtype):
 
 
 def test_ffn_refuses_what_it_cannot_run():
-    """loud failures, no fallback: half precision, an activation the kernels do not have, a plug-in matmul op"""
+    """loud failures, no fallback: double precision, bfloat16 activations into float16 weights, an activation the kernels
+    do not have, an input of the wrong width"""
     ffn = lt.LeanFFN(256, 512).to(DEV)
     with pytest.raises(TypeError):
-        ffn.half()(torch.zeros(4, 256, device=DEV, dtype=torch.float16))
+        ffn.double()(torch.zeros(4, 256, device=DEV, dtype=torch.float64))
+    with pytest.raises(TypeError):
+        ffn.half()(torch.zeros(4, 256, device=DEV, dtype=torch.bfloat16))
     with pytest.raises((NotImplementedError, ValueError, KeyError, RuntimeError)):
         lt.LeanFFN(256, 512, activation=lambda t: t * 2).to(DEV)(torch.zeros(4, 256, device=DEV))
     with pytest.raises(RuntimeError):

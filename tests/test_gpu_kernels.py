@@ -22,9 +22,10 @@ GOLDEN = np.load(os.path.join(os.path.dirname(__file__), "golden", "blocksparse_
 
 def _gemm(a, b, a_kmajor, b_kmajor, m, n, k, c_dtype, force_generic):
     c = torch.empty(m, n, dtype=c_dtype, device=DEV)
-    nat.check(nat.lib().lt_gemm(nat.dtype_code(a.dtype), m, n, k, nat.ptr(a), int(a_kmajor), nat.ptr(b), int(b_kmajor),
-                                nat.dtype_code(c_dtype), nat.ptr(c), int(force_generic), nat.current_stream(c.device)),
-              "lt_gemm")
+    lib = nat.lib(a.dtype, c_dtype)
+    nat.check(lib.lt_gemm(nat.dtype_code(a.dtype), m, n, k, nat.ptr(a), int(a_kmajor), nat.ptr(b), int(b_kmajor),
+                          nat.dtype_code(c_dtype), nat.ptr(c), int(force_generic), nat.current_stream(c.device)),
+              "lt_gemm", lib)
     return c
 
 

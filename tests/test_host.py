@@ -164,10 +164,15 @@ def test_library_loads_and_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "leanffn.h")).read()
     declared = set(re.findall(r"\b(lt_[a-z0-9_]+)\s*\(", header))
     assert declared == set(nat.EXPORTED_SYMBOLS), declared ^ set(nat.EXPORTED_SYMBOLS)
-    lib = nat.lib()
-    for name in declared:
-        assert hasattr(lib, name), name
-    assert lib.lt_version().decode().startswith("libleanffn")
+    for dtype, half in ((torch.bfloat16, "bf16"), (torch.float16, "fp16")):  # the library and its float16 twin
+        lib = nat.lib(dtype)
+        for name in declared:
+            assert hasattr(lib, name), name
+        version = lib.lt_version().decode()
+        assert version.startswith("libleanffn") and half in version, version
+    assert nat.lib() is nat.lib(torch.float32) is nat.lib(torch.bfloat16) is not nat.lib(torch.float16)
+    with pytest.raises(TypeError, match="one 16-bit type"):
+        nat.lib(torch.float16, torch.bfloat16)
 
 
 def test_struct_layouts_match_header_sizes():
