@@ -506,7 +506,7 @@ def test_custom_grad_switch_and_partial_grads():
     assert_close(g3[0], g1[0], torch.float32, "dx under checkpoint")
 
 
-def _headline(hidden, inter, gated, std, dropout, shape, seed=0):
+def _headline(hidden, inter, gated, std, dropout, shape, seed=0, dtype=torch.bfloat16):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(*shape, hidden, generator=g)
     n1 = 2 * inter if gated else inter
@@ -517,30 +517,30 @@ def _headline(hidden, inter, gated, std, dropout, shape, seed=0):
         ffn.i2h_proj.bias.zero_()
         ffn.h2o_proj.bias.zero_()
     dy = torch.randn(*shape, hidden, generator=g)
-    return ffn.to(DEV).to(torch.bfloat16), x, dy
+    return ffn.to(DEV).to(dtype), x, dy
 
 
-def _full_size_checks(ffn, x, dy, mask_p):
+def _full_size_checks(ffn, x, dy, mask_p, dtype=torch.bfloat16):
     tokens, hidden = x.shape[0] * x.shape[1], x.shape[-1]
     torch.cuda.manual_seed(0)
     seed, offset = generator_position(DEV)
     y, dx, g = _run_module(ffn, x.to(DEV), dy.to(DEV))
     mask = dropout_mask(tokens, hidden, mask_p, seed, offset, torch.device(DEV)) if mask_p > 0 else None
-    # (1) the oracle, evaluated in fp32 on the GPU, on the bf16-rounded weights
+    # (1) the oracle, evaluated in fp32 on the GPU, on the rounded weights
     p = oracle_params(ffn, DEV)
     y_ref, dx_ref, g_ref = run_oracle(p, x.float().to(DEV), dy.float().to(DEV), mask)
-    assert_close(y, y_ref, torch.bfloat16, "y")
-    assert_close(dx, dx_ref, torch.bfloat16, "dx")
+    assert_close(y, y_ref, dtype, "y")
+    assert_close(dx, dx_ref, dtype, "dx")
     for i, (a, b) in enumerate(zip(g, g_ref)):
-        assert_close(a, b, torch.bfloat16, f"param grad {i}")
+        assert_close(a, b, dtype, f"param grad {i}")
     del p, y_ref, dx_ref, g_ref
     # (2) rows are independent: 128 rows through the oracle on the CPU
     rows = torch.randperm(tokens, generator=torch.Generator().manual_seed(1))[:128]
     p_cpu = oracle_params(ffn, "cpu")
     x2, dy2 = x.float().reshape(tokens, hidden)[rows], dy.float().reshape(tokens, hidden)[rows]
     y_cpu, dx_cpu, _ = run_oracle(p_cpu, x2, dy2, None if mask is None else mask.cpu()[rows])
-    assert_close(y.reshape(tokens, hidden)[rows.to(DEV)], y_cpu, torch.bfloat16, "y rows")
-    assert_close(dx.reshape(tokens, hidden)[rows.to(DEV)], dx_cpu, torch.bfloat16, "dx rows")
+    assert_close(y.reshape(tokens, hidden)[rows.to(DEV)], y_cpu, dtype, "y rows")
+    assert_close(dx.reshape(tokens, hidden)[rows.to(DEV)], dx_cpu, dtype, "dx rows")
     # (3) weight gradients are sums over tokens: two halves of the batch add up to the whole (no dropout in this check,
     #     each half draws its own stream)
     if mask is None:
@@ -549,7 +549,7 @@ def _full_size_checks(ffn, x, dy, mask_p):
         _, _, ga = _run_module(ffn, xf[:half].to(DEV), dyf[:half].to(DEV))
         _, _, gb = _run_module(ffn, xf[half:].to(DEV), dyf[half:].to(DEV))
         for i, (whole, a, b) in enumerate(zip(g, ga, gb)):
-            assert_close(whole.float(), a.float() + b.float(), torch.bfloat16, f"additivity of param grad {i}")
+            assert_close(whole.float(), a.float() + b.float(), dtype, f"additivity of param grad {i}")
 
 
 def test_config2_bf16_full_size():

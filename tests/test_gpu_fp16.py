@@ -12,7 +12,7 @@ from conftest import assert_close, rel_err
 from helpers import dropout_mask, generator_position
 from lean_transformer_amd import _native as nat
 from lean_transformer_amd.utils import ACT2FN
-from test_gpu_ffn import _compare
+from test_gpu_ffn import _compare, _full_size_checks, _headline
 from test_gpu_ffn_bf16_paths import _dense_from_native, _randomise_small_vectors
 from test_gpu_kernels import _gemm, _operands
 
@@ -181,3 +181,10 @@ def test_fp16_autocast_with_fp32_master_weights():
     assert_close(y, yh.float(), F16, "y against the fp16 module")
     for i, (a, b) in enumerate(zip(grads, gh)):
         assert_close(a, b.float(), F16, f"grad {i} against the fp16 module")
+
+
+def test_config3_fp16_full_size():
+    """benchmark config 3 in float16: hidden 4096, intermediate 16384, GeGLU, x [2, 2048, 4096], weights ~N(0, 0.01); the
+    oracle in fp32 on the GPU, 128 rows through the CPU oracle, weight gradients additive over token halves"""
+    ffn, x, dy = _headline(4096, 16384, True, 0.01, 0.0, (2, 2048), dtype=F16)
+    _full_size_checks(ffn, x, dy, 0.0, dtype=F16)
