@@ -400,7 +400,7 @@ struct BwdScratch {
   void* hid;         // [T, I]
   void* dpre;        // [T, N1]
   void* u;           // [T, H]
-  float* du;         // [T, H] fp32
+  void* du;          // [T, H] compute dtype (as the reference's autocast matmul leaves it)
   void* ln_ws;
   size_t ln_ws_bytes;
   float* act_colsum;  // [ceil(T / 64), N1]: partial column sums of dpre from the epilogue that writes it
@@ -417,7 +417,7 @@ void plan_backward(const lt_ffn_desc& d, Bump& ws, BwdScratch& s) {
   s.hid = ws.take((size_t)T * d.intermediate * e);
   s.dpre = ws.take((size_t)T * n1 * e);
   s.u = ws.take((size_t)T * d.hidden * e);
-  s.du = (float*)ws.take((size_t)T * d.hidden * sizeof(float));
+  s.du = ws.take((size_t)T * d.hidden * e);
   s.ln_ws_bytes = lt_ln_backward_workspace(T, d.hidden);
   s.ln_ws = ws.take(s.ln_ws_bytes);
   s.act_colsum = (float*)ws.take((size_t)((T + 63) / 64) * n1 * sizeof(float));
@@ -551,17 +551,17 @@ extern "C" int lt_ffn_backward(const lt_ffn_desc* desc, const void* x, const voi
     i2h_grads.bias = nullptr;
   }
 
-  // up-projection backward on the recomputed LayerNorm output; du in fp32
+  // up-projection backward on the recomputed LayerNorm output; du in the compute dtype
   LT_TRY(lt_ln_forward(T, (int)H, d.ln_eps, io, x, d.ln_weight, d.ln_bias, cdt, s.u, nullptr, io, nullptr, nullptr, false,
                        stream));
   const bool need_du = grads->dx || grads->ln_weight;
   {
-    EpiParams e = epi_store_params(s.du, H, LT_F32, nullptr);
+    EpiParams e = epi_store_params(s.du, H, cdt, nullptr);
     LT_TRY(linear_backward_impl(d.i2h, T, cdt, s.u, s.dpre, saved->i2h_lowrank_hid, need_du ? EPI_STORE : -1, e,
                                 i2h_grads, s.i2h, io, stream));
   }
   if (need_du) {
-    LT_TRY(lt_ln_backward(T, (int)H, io, x, saved->ln_stats, d.ln_weight, LT_F32, s.du, io, d.residual ? dy : nullptr,
+    LT_TRY(lt_ln_backward(T, (int)H, io, x, saved->ln_stats, d.ln_weight, cdt, s.du, io, d.residual ? dy : nullptr,
                           grads->dx, grads->ln_weight, grads->ln_bias, s.ln_ws, s.ln_ws_bytes, stream, &reduces));
   }
   return lt_colreduce_flush(reduces, stream);
