@@ -8,7 +8,8 @@ K steps are timed by wall clock; the same K steps are then repeated with a HIP e
 (recorded by the library on the launch stream) and `roofline` is computed from the GEMM launches of that pass;
 `cpu_baseline` times the CPU oracle (tests' checker, not the product) on a bounded sample of the same workload.
 The default run also measures configurations 2, 4 and 4 with the reference's default layout (c4t: stretch=False), about a
-second of GPU time each, and reports them under `extra_configs` of the same line;
+second of GPU time each, and reports them under `extra_configs` of the same line; `--config c3h` is configuration 3 in
+float16 on the library's float16 build;
 `--config c5` times the full GPT train step of configuration 5 (the stock-PyTorch model of tests/gpt_harness.py around the
 FFN kernels).
 """
